@@ -3,14 +3,23 @@ from ..registry import architecture
 from ..status import EFORMAT, ENOTSUP, fail
 from .reader import KeyReader, config_path, read_json_file
 from .qwen2 import Qwen2Config
+from .goridra import GoridraConfig
+
+
+def architecture_name(obj, origin="config.json"):
+    """The name that chooses the model class: the first of ``architectures``, or the string ``architecture``."""
+    r = KeyReader(obj, origin)
+    if not r.has("architectures") and r.has("architecture"):
+        return r.string("architecture")
+    names = r.str_list("architectures")
+    if not names:
+        fail(EFORMAT, f"{origin}: key 'architectures' is empty")
+    return names[0]
 
 
 def config_from_dict(obj, origin="config.json"):
-    """The typed configuration for ``obj['architectures'][0]``, by the registry."""
-    names = KeyReader(obj, origin).str_list("architectures")
-    if not names:
-        fail(EFORMAT, f"{origin}: key 'architectures' is empty")
-    config_cls, _ = architecture(names[0])
+    """The typed configuration for the architecture that ``obj`` names, by the registry."""
+    config_cls, _ = architecture(architecture_name(obj, origin))
     return config_cls.from_dict(obj, origin)
 
 
@@ -23,13 +32,11 @@ def apply_model_options(obj, options, origin="config.json"):
     options = {k: v for k, v in (options or {}).items() if v is not None}
     if not options:
         return obj
-    names = KeyReader(obj, origin).str_list("architectures")
-    if not names:
-        fail(EFORMAT, f"{origin}: key 'architectures' is empty")
-    config_cls, _ = architecture(names[0])
+    name = architecture_name(obj, origin)
+    config_cls, _ = architecture(name)
     hook = getattr(config_cls, "apply_options", None)
     if hook is None:
-        fail(ENOTSUP, f"architecture '{names[0]}' takes no model options (given: {', '.join(sorted(options))})")
+        fail(ENOTSUP, f"architecture '{name}' takes no model options (given: {', '.join(sorted(options))})")
     return hook(obj, options)
 
 
@@ -40,4 +47,4 @@ def read_config(model_dir, options=None):
     return config_from_dict(apply_model_options(read_json_file(path), options, path), path)
 
 
-__all__ = ["KeyReader", "Qwen2Config", "apply_model_options", "config_from_dict", "read_config", "read_json_file"]
+__all__ = ["GoridraConfig", "KeyReader", "Qwen2Config", "architecture_name", "apply_model_options", "config_from_dict", "read_config", "read_json_file"]

@@ -82,7 +82,8 @@ int hfa_attention_prompt_rows(void);
 // Softmax attention of each token's query heads over its request's cached keys and values
 // (src/model.c:499-528). Key j of the request in slot s lies in cache row
 // block_table[s, j / page_tokens] * page_tokens + j % page_tokens. A key is visible to the
-// query at position p iff j <= p and (window == 0 or p - j < window). q_start[n_seqs + 1] gives
+// query at position p iff j <= p and (window == 0 or p - j < window) and (mask_chunk == 0 or
+// j / mask_chunk == p / mask_chunk: a mask by runs of mask_chunk positions counted from 0). q_start[n_seqs + 1] gives
 // each request's run of tokens (consecutive positions of one slot); max_q_len and max_seq_len
 // bound the runs and the positions. Key rows are kv_width wide with head_dim values a head, value rows
 // v_width with v_head_dim a head; out has v_head_dim values per query head. bf16 with one head size for
@@ -96,7 +97,7 @@ int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, 
                         int kv_width, int v_width, const int* block_table, int max_blocks, const int* token_slot,
                         const int* positions, const int* q_start, int n_seqs, int max_q_len, int max_seq_len,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
-                        int page_tokens, int window, float scale, const float* slopes, void* workspace,
+                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, void* workspace,
                         size_t workspace_bytes, int force_plain, hipStream_t stream);
 
 // Decoded tokens (one a request) whose queries, new keys and new values are still the 32-bit rows [q | k | v] that
@@ -111,8 +112,46 @@ int hfa_decode_attention_supports(int n_heads, int n_kv_heads, int head_dim, int
 int hfa_decode_attention(const float* raw, int ld_raw, const float* cos_sin, void* k_cache, void* v_cache, int kv_width,
                          const int* slot_map, const int* block_table, int max_blocks, const int* token_slot,
                          const int* positions, const int* q_start, int n_seqs, int max_seq_len, void* out, int ldo,
-                         int n_heads, int n_kv_heads, int head_dim, int page_tokens, int window, float scale,
+                         int n_heads, int n_kv_heads, int head_dim, int page_tokens, int window, int mask_chunk, float scale,
                          void* workspace, size_t workspace_bytes, hipStream_t stream);
+
+// Layer norm: out[r, :] = (x[rows ? rows[r] : r, :] - mean) / sqrt(var + eps) * w + b (b null: no shift), var the mean
+// squared deviation, all in fp32. With splits > 0 (and no rows) a deferred product's partial sums
+// ([splits][x_rows][width]) and partial_bias are first added into x, as in hfa_rmsnorm.
+int hfa_layernorm(float* x, const float* w, const float* b, void* out, int out_dtype, const int* rows, int n_rows,
+                  int width, float eps, const float* partial, int splits, const float* partial_bias, int x_rows,
+                  hipStream_t stream);
+
+// out[r, c] = act(in[r, c]) for rows of `width` values with strides ldi and ldo, computed in fp32:
+// the exact gelu 0.5 z (1 + erf(z / sqrt 2)), its tanh form, or relu(z)^2.
+#define HFA_ACT_NONE 0
+#define HFA_ACT_GELU_ERF 1
+#define HFA_ACT_GELU_TANH 2
+#define HFA_ACT_RELU2 3
+int hfa_activation(const void* in, int ldi, void* out, int ldo, int dtype, int n_rows, int width, int kind,
+                   hipStream_t stream);
+
+// x <- cap * tanh(x / cap) on fp32 rows, in place (logits that a model squashes).
+int hfa_softcap(float* x, int ld, int n_rows, int width, float cap, hipStream_t stream);
+
+// Mixture of experts (moe.hip). hfa_moe_route: fp32 router logits [n_tokens, n_experts] -> ids and weights
+// [n_tokens, top]; scoring 0 = softmax over all experts, 1 = logistic per expert; experts form n_groups equal runs of
+// neighbours of which the `keep` best (by their best expert) may be chosen from; weights = score (/ sum of the chosen
+// + 1e-20 if renorm) * out_scale. hfa_moe_plan puts the n_pairs = n_tokens * top pairs in expert order (row_pair) and
+// lists tiles of at most tile_rows rows of one expert (tiles: 3 ints a tile, room for n_pairs / tile_rows + n_experts;
+// *n_tiles on the device). hfa_moe_gemm: for every row r of the plan, out[o(r), :] = act(a[s(r), :] . w[e(r)]^T)
+// (* pair_scale[pair] if given); w is [n_experts][N][K]; s(r) = row_pair[r] / a_div if a_div > 0 else r; o(r) =
+// row_pair[r] if out_by_pair else r. tile_rows must be what hfa_moe_tile_rows gave for the plan.
+// hfa_moe_combine: x[t, :] += sum_k y[t * top + k, :].
+int hfa_moe_route(const float* logits, int ld, int n_tokens, int n_experts, int top, int n_groups, int keep,
+                  int scoring, int renorm, float out_scale, int* ids, float* weights, hipStream_t stream);
+int hfa_moe_plan(const int* ids, int n_pairs, int n_experts, int tile_rows, int* row_pair, int* tiles, int* n_tiles,
+                 hipStream_t stream);
+int hfa_moe_tile_rows(int dtype, int n_pairs, int n_experts, int N, int K);
+int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const void* w, const int* row_pair, const int* tiles,
+                 const int* n_tiles, int max_tiles, int tile_rows, void* out, int ldo, int out_dtype, int out_by_pair,
+                 const float* pair_scale, int act, int N, int K, int force_plain, hipStream_t stream);
+int hfa_moe_combine(const float* y, float* x, int n_tokens, int top, int width, hipStream_t stream);
 
 // out[t, i] = silu(gate_up[t, i]) * gate_up[t, width + i].  (src/model.c:532-538)
 int hfa_swiglu(const void* gate_up, void* out, int dtype, int n_tokens, int width, hipStream_t stream);

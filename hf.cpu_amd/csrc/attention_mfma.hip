@@ -76,7 +76,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     const uint16_t* __restrict__ q, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, int kvw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
-    int ldo, float* __restrict__ partial, int H, int psh, int window, float scale_log2e, int tpt, int cpt,
+    int ldo, float* __restrict__ partial, int H, int psh, int window, int mask_chunk, float scale_log2e, int tpt, int cpt,
     int chunk_keys, int n_chunks, int one_tile_each, const float* __restrict__ raw, int ld_raw,
     const float* __restrict__ cs, const int* __restrict__ slot_map, int G) {
     constexpr int D = NDB * 32, KS = D / 16;
@@ -110,14 +110,14 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     const int my_head = g * cpt + (col_ok ? col % cpt : 0);
     const int pos = positions[my_tok];
     const int pos_first = positions[t0], hi = positions[t_end - 1];
-    int k_begin = window > 0 && pos_first - window + 1 > 0 ? pos_first - window + 1 : 0;
+    int k_begin = first_visible(pos_first, window, mask_chunk);
     int k_end = hi;
     if (SPLIT) {
         k_begin = k_begin > chunk * chunk_keys ? k_begin : chunk * chunk_keys;
         k_end = k_end < (chunk + 1) * chunk_keys - 1 ? k_end : (chunk + 1) * chunk_keys - 1;
     }
     // visible keys of this lane's column: [vlo, vhi]
-    int vlo = window > 0 && pos - window + 1 > k_begin ? pos - window + 1 : k_begin;
+    int vlo = first_visible(pos, window, mask_chunk) > k_begin ? first_visible(pos, window, mask_chunk) : k_begin;
     int vhi = col_ok ? (pos < k_end ? pos : k_end) : -1;
     const int* bt = block_table + (size_t)token_slot[t0] * max_blocks;
 
@@ -479,7 +479,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     const uint16_t* __restrict__ q, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc, int kvw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
-    int ldo, int psh, int window, float scale_log2e, int tpt, int cpt, int n_tiles, int pair_from,
+    int ldo, int psh, int window, int mask_chunk, float scale_log2e, int tpt, int cpt, int n_tiles, int pair_from,
     float* __restrict__ partial, int H, int chunk_keys, int n_chunks) {
     constexpr int D = NDB * 32, KS = D / 16, KROW = D + 8;
     const int P = 1 << psh;                                // tokens per page, a power of two
@@ -530,7 +530,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     const int pos = positions[my_tok];
     const int pos_first = positions[t0];
     int hi = positions[t_end - 1];
-    int k_begin = window > 0 && pos_first - window + 1 > 0 ? pos_first - window + 1 : 0;
+    int k_begin = first_visible(pos_first, window, mask_chunk);
     // With n_chunks > 1 the block takes the keys of chunk blockIdx.z only (chunk_keys is a multiple
     // of the key block) and leaves maximum, sum and unscaled output for attn_merge_kernel; a chunk
     // that holds none of the tile's keys leaves an empty record.
@@ -539,7 +539,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
         k_begin = k_begin > c_lo ? k_begin : c_lo;
         hi = hi < c_hi ? hi : c_hi;
     }
-    const int vlo = window > 0 && pos - window + 1 > k_begin ? pos - window + 1 : k_begin;
+    const int vlo = first_visible(pos, window, mask_chunk) > k_begin ? first_visible(pos, window, mask_chunk) : k_begin;
     const int vhi = col_ok ? (pos < hi ? pos : hi) : -1;
     const int* bt = block_table + (size_t)token_slot[t0] * max_blocks;
 
@@ -886,7 +886,7 @@ static int launch_ndb(const AttnArgs& a, int tiles, int tpt, int cpt, int chunk_
 #define ATTN_ARGS(PARTIAL)                                                                                              \
     (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,      \
         a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo, PARTIAL, a.n_heads,         \
-        page_shift(a.page_tokens), a.window, sl, tpt, cpt, chunk_keys, n_chunks, a.max_q_len <= tpt, a.raw, a.ld_raw,      \
+        page_shift(a.page_tokens), a.window, a.mask_chunk, sl, tpt, cpt, chunk_keys, n_chunks, a.max_q_len <= tpt, a.raw, a.ld_raw,      \
         a.cos_sin, a.slot_map, a.n_kv_heads
     if (a.raw) {
         if (n_chunks > 1) attn_mfma_kernel<NDB, true, true><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS((float*)a.workspace));
@@ -942,13 +942,13 @@ static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
         attn_prefill_kernel<NDB, true><<<grid, 4 * WAVE, 0, a.stream>>>(
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
             a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
+            page_shift(a.page_tokens), a.window, a.mask_chunk, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
             (float*)a.workspace, a.n_heads, chunk_keys, n_chunks);
     else
         attn_prefill_kernel<NDB, false><<<grid, 4 * WAVE, 0, a.stream>>>(
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
             a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
-            page_shift(a.page_tokens), a.window, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
+            page_shift(a.page_tokens), a.window, a.mask_chunk, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
             (float*)a.workspace, a.n_heads, chunk_keys, n_chunks);
     HFA_LAUNCH_CHECK("attn_prefill");
     if (n_chunks > 1) {
@@ -986,7 +986,8 @@ int attn_mfma_launch(const AttnArgs& a) {
     const int tiles = a.max_q_len <= tpt ? a.n_seqs : (a.n_tokens + tpt - 1) / tpt + a.n_seqs;
     // Few waves and long contexts: cut the keys into chunks so that the machine is full.
     const long waves = (long)(a.max_q_len <= tpt ? a.n_seqs : (a.n_tokens + tpt - 1) / tpt) * a.n_kv_heads;
-    const int span = a.window > 0 && a.window + a.max_q_len < a.max_seq_len ? a.window + a.max_q_len : a.max_seq_len;
+    int span = a.window > 0 && a.window + a.max_q_len < a.max_seq_len ? a.window + a.max_q_len : a.max_seq_len;
+    if (a.mask_chunk > 0 && a.mask_chunk + a.max_q_len < span) span = a.mask_chunk + a.max_q_len;      // a masking chunk bounds the keys as a window does
     int n_chunks = 1, chunk_keys = a.max_seq_len;
     // How many waves in all is a measured choice. Head size 128 (7B shape): 512; with 1,024 a step took 1.3 % longer
     // at 64 sequences and 4.5 % longer at 8 sequences of 16,384 tokens, with 256 more than that. Head size 64 (0.5B

@@ -1,0 +1,371 @@
+// Mixture of experts: the router's choice, the plan of a step (which rows go to which expert), the products of all
+// experts in one launch, and the weighted sum into the residual stream.
+//
+//   hfa_moe_route    fp32 router logits -> the chosen experts of each token and their weights
+//   hfa_moe_plan     the (token, choice) pairs put in the order of their experts, and the tiles of rows that the
+//                    products walk: nothing of a step's routing is known to the host
+//   hfa_moe_gemm     out[row] = act(a[src(row)] . w[expert of row]^T), one block a tile of rows of one expert
+//   hfa_moe_combine  x[t] += sum over the token's choices, in the order of the choices
+//
+// A row's result depends on its own operands only and is summed over K in one fixed order, so neither the rest of the
+// batch nor the place that a pair got inside its expert's run changes it.
+#include "api.h"
+#include "common.h"
+
+#define MOE_MAX_EXPERTS 1024
+
+// ---- router -----------------------------------------------------------------------------
+// The better of two candidates: the larger score, the lower index among equals.
+__device__ __forceinline__ void better(float& v, int& i, float v2, int i2) {
+    if (v2 > v || (v2 == v && i2 < i)) { v = v2; i = i2; }
+}
+__device__ __forceinline__ void wave_best(float& v, int& i) {
+#pragma unroll
+    for (int off = WAVE / 2; off > 0; off >>= 1) {
+        const float v2 = __shfl_xor(v, off, WAVE);
+        const int i2 = __shfl_xor(i, off, WAVE);
+        better(v, i, v2, i2);
+    }
+}
+
+// One wave a token. score = softmax over all experts (or the logistic function of each logit, `scoring` 1); experts
+// form n_groups runs of neighbours, a run scores as its best expert, and only experts of the `keep` best runs can
+// be chosen; the `top` best of those are chosen, and weigh score / (sum of the chosen scores + 1e-20) if `renorm`,
+// else their score; times `out_scale`.
+__global__ __launch_bounds__(WAVE) void moe_route_kernel(const float* __restrict__ logits, int ld, int E, int top,
+                                                        int n_groups, int keep, int scoring, int renorm, float out_scale,
+                                                        int* __restrict__ ids, float* __restrict__ weights) {
+    __shared__ float s[MOE_MAX_EXPERTS];
+    __shared__ float gs[MOE_MAX_EXPERTS];
+    __shared__ unsigned char open_s[MOE_MAX_EXPERTS];        // per group: may be chosen from
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const float* z = logits + (size_t)t * ld;
+    if (scoring == 0) {
+        float m = -INFINITY;
+        for (int e = lane; e < E; e += WAVE) m = fmaxf(m, z[e]);
+        m = wave_max(m);
+        float sum = 0.f;
+        for (int e = lane; e < E; e += WAVE) {
+            const float p = expf(z[e] - m);
+            s[e] = p;
+            sum += p;
+        }
+        sum = wave_sum(sum);
+        for (int e = lane; e < E; e += WAVE) s[e] = s[e] / sum;
+    } else {
+        for (int e = lane; e < E; e += WAVE) s[e] = 1.0f / (1.0f + expf(-z[e]));
+    }
+    __syncthreads();
+    const int per = E / n_groups;
+    for (int g = lane; g < n_groups; g += WAVE) {
+        float b = -INFINITY;
+        for (int e = g * per; e < (g + 1) * per; e++) b = fmaxf(b, s[e]);
+        gs[g] = b;
+        open_s[g] = keep >= n_groups ? 1 : 0;
+    }
+    __syncthreads();
+    if (keep < n_groups) {
+        for (int r = 0; r < keep; r++) {
+            float bv = -INFINITY;
+            int bi = 0x7fffffff;
+            for (int g = lane; g < n_groups; g += WAVE)
+                if (!open_s[g]) better(bv, bi, gs[g], g);
+            wave_best(bv, bi);
+            if (lane == 0 && bi < n_groups) open_s[bi] = 1;
+            __syncthreads();
+        }
+    }
+    float chosen_sum = 0.f;
+    for (int r = 0; r < top; r++) {
+        float bv = -INFINITY;
+        int bi = 0x7fffffff;
+        for (int e = lane; e < E; e += WAVE)
+            if (open_s[e / per] && s[e] >= 0.f) better(bv, bi, s[e], e);
+        wave_best(bv, bi);
+        if (bi >= E) { bi = 0; bv = 0.f; }                   // fewer open experts than choices: weight nothing
+        else if (lane == 0) s[bi] = -1.f;                    // taken
+        if (lane == 0) {
+            ids[(size_t)t * top + r] = bi;
+            weights[(size_t)t * top + r] = bv;
+        }
+        chosen_sum += bv;
+        __syncthreads();
+    }
+    if (lane < top) {
+        const float wv = weights[(size_t)t * top + lane];
+        weights[(size_t)t * top + lane] = (renorm ? wv / (chosen_sum + 1e-20f) : wv) * out_scale;
+    }
+}
+
+extern "C" int hfa_moe_route(const float* logits, int ld, int n_tokens, int n_experts, int top, int n_groups, int keep,
+                             int scoring, int renorm, float out_scale, int* ids, float* weights, hipStream_t stream) {
+    HFA_REQUIRE(logits && ids && weights && n_tokens > 0, "moe_route: bad arguments");
+    HFA_REQUIRE(n_experts > 0 && n_experts <= MOE_MAX_EXPERTS && ld >= n_experts, "moe_route: %d experts (at most %d)", n_experts,
+                MOE_MAX_EXPERTS);
+    HFA_REQUIRE(top > 0 && top <= WAVE && top <= n_experts, "moe_route: %d choices of %d experts (at most %d)", top, n_experts, WAVE);
+    HFA_REQUIRE(n_groups > 0 && n_experts % n_groups == 0 && keep > 0 && keep <= n_groups,
+                "moe_route: %d experts do not form %d equal groups of which %d are kept", n_experts, n_groups, keep);
+    HFA_REQUIRE(scoring == 0 || scoring == 1, "moe_route: unknown scoring %d", scoring);
+    moe_route_kernel<<<n_tokens, WAVE, 0, stream>>>(logits, ld, n_experts, top, n_groups, keep, scoring, renorm, out_scale, ids,
+                                                    weights);
+    HFA_LAUNCH_CHECK("moe_route");
+    return 0;
+}
+
+// ---- plan -------------------------------------------------------------------------------
+// Pair p = token * top + choice goes to expert ids[p]. row_pair[r] = the pair in row r of the expert-ordered rows;
+// tiles[3 i ..] = (expert, first row, rows) of tile i, tiles of at most tile_rows rows of one expert; *n_tiles their
+// number (at most n_pairs / tile_rows + n_experts). One block.
+__global__ __launch_bounds__(1024) void moe_plan_kernel(const int* __restrict__ ids, int n_pairs, int E, int tile_rows,
+                                                       int* __restrict__ row_pair, int* __restrict__ tiles,
+                                                       int* __restrict__ n_tiles) {
+    __shared__ int count[MOE_MAX_EXPERTS];
+    __shared__ int start[MOE_MAX_EXPERTS];
+    __shared__ int tile0[MOE_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) atomicAdd(&count[ids[p]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int rows = 0, nt = 0;
+        for (int e = 0; e < E; e++) {
+            start[e] = rows;
+            tile0[e] = nt;
+            rows += count[e];
+            nt += (count[e] + tile_rows - 1) / tile_rows;
+        }
+        *n_tiles = nt;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        const int c = count[e];
+        for (int i = 0, r = 0; r < c; i++, r += tile_rows) {
+            int* tl = tiles + 3 * (tile0[e] + i);
+            tl[0] = e;
+            tl[1] = start[e] + r;
+            tl[2] = c - r < tile_rows ? c - r : tile_rows;
+        }
+    }
+    __syncthreads();
+    // Where a pair lands inside its expert's run is whatever order the atomics give: a row's result does not depend
+    // on its place (see the head of this file).
+    for (int p = threadIdx.x; p < n_pairs; p += blockDim.x) row_pair[atomicAdd(&start[ids[p]], 1)] = p;
+}
+
+extern "C" int hfa_moe_plan(const int* ids, int n_pairs, int n_experts, int tile_rows, int* row_pair, int* tiles,
+                            int* n_tiles, hipStream_t stream) {
+    HFA_REQUIRE(ids && row_pair && tiles && n_tiles && n_pairs > 0 && tile_rows > 0, "moe_plan: bad arguments");
+    HFA_REQUIRE(n_experts > 0 && n_experts <= MOE_MAX_EXPERTS, "moe_plan: %d experts (at most %d)", n_experts, MOE_MAX_EXPERTS);
+    int threads = n_pairs >= 1024 ? 1024 : (n_pairs + WAVE - 1) / WAVE * WAVE;
+    moe_plan_kernel<<<1, threads, 0, stream>>>(ids, n_pairs, n_experts, tile_rows, row_pair, tiles, n_tiles);
+    HFA_LAUNCH_CHECK("moe_plan");
+    return 0;
+}
+
+// ---- the experts' products ----------------------------------------------------------------
+__device__ __forceinline__ float moe_act(int act, float z) {
+    if (act == HFA_ACT_RELU2) { const float r = fmaxf(z, 0.f); return r * r; }
+    if (act == HFA_ACT_GELU_ERF) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+    if (act == HFA_ACT_GELU_TANH) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+    return z;
+}
+
+// Plain form, any dtype and shape: a tile of up to 32 rows x 64 columns a block, operands staged through LDS 32 k at a
+// time, every output summed over k in ascending order by one thread.
+#define PM 32
+#define PN 64
+#define PK 32
+template <typename T, typename TO>
+__global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
+    const T* __restrict__ a, int lda, int a_div, const T* __restrict__ w, const int* __restrict__ row_pair,
+    const int* __restrict__ tiles, const int* __restrict__ n_tiles, TO* __restrict__ out, int ldo, int out_by_pair,
+    const float* __restrict__ pair_scale, int act, int N, int K) {
+    if ((int)blockIdx.x >= *n_tiles) return;
+    __shared__ float a_s[PM][PK + 1];
+    __shared__ float w_s[PN][PK + 1];
+    __shared__ int src_s[PM], pair_s[PM];
+    const int e = tiles[3 * blockIdx.x], r0 = tiles[3 * blockIdx.x + 1], nr = tiles[3 * blockIdx.x + 2];
+    const int n0 = blockIdx.y * PN, tid = threadIdx.x;
+    if (tid < PM) {
+        const int pair = row_pair[r0 + (tid < nr ? tid : 0)];
+        pair_s[tid] = pair;
+        src_s[tid] = a_div > 0 ? pair / a_div : r0 + (tid < nr ? tid : 0);
+    }
+    __syncthreads();
+    const T* we = w + (size_t)e * N * K;
+    const int col = tid & (PN - 1), rg = tid / PN;          // 4 row groups of 8 rows
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; i++) acc[i] = 0.f;
+    for (int k0 = 0; k0 < K; k0 += PK) {
+        for (int i = tid; i < PM * PK; i += 256) {
+            const int r = i / PK, k = i % PK;
+            a_s[r][k] = k0 + k < K ? to_f32(a[(size_t)src_s[r] * lda + k0 + k]) : 0.f;
+        }
+        for (int i = tid; i < PN * PK; i += 256) {
+            const int n = i / PK, k = i % PK;
+            w_s[n][k] = (k0 + k < K && n0 + n < N) ? to_f32(we[(size_t)(n0 + n) * K + k0 + k]) : 0.f;
+        }
+        __syncthreads();
+        const int kn = K - k0 < PK ? K - k0 : PK;
+        for (int k = 0; k < kn; k++) {
+            const float wv = w_s[col][k];
+#pragma unroll
+            for (int i = 0; i < 8; i++) acc[i] = fmaf(a_s[rg * 8 + i][k], wv, acc[i]);
+        }
+        __syncthreads();
+    }
+    if (n0 + col >= N) return;
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        const int r = rg * 8 + i;
+        if (r >= nr) continue;
+        float v = moe_act(act, acc[i]);
+        if (pair_scale) v *= pair_scale[pair_s[r]];
+        const size_t orow = out_by_pair ? (size_t)pair_s[r] : (size_t)(r0 + r);
+        out[orow * ldo + n0 + col] = from_f32<TO>(v);
+    }
+}
+
+// Matrix-core form (bf16 operands, K a multiple of 16, N of 32): a block of four waves owns 32 RM rows x 128 CN columns
+// of one expert, a wave 32 RM x 32 CN of them. Both operands are K-contiguous, so a lane's 8 consecutive k of one row
+// are one 16-byte load straight into the operand registers of v_mfma_f32_32x32x16_bf16; the four waves of a block read
+// the same rows of `a`, which the CU's cache serves after the first.
+typedef __bf16 mbf16x8 __attribute__((ext_vector_type(8)));
+typedef float mfloatx16 __attribute__((ext_vector_type(16)));
+union MFrag {
+    uint4 u;
+    mbf16x8 v;
+};
+
+template <int RM, int CN, typename TO>
+__global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
+    const uint16_t* __restrict__ a, int lda, int a_div, const uint16_t* __restrict__ w, const int* __restrict__ row_pair,
+    const int* __restrict__ tiles, const int* __restrict__ n_tiles, TO* __restrict__ out, int ldo, int out_by_pair,
+    const float* __restrict__ pair_scale, int act, int N, int K) {
+    if ((int)blockIdx.x >= *n_tiles) return;
+    const int e = tiles[3 * blockIdx.x], r0 = tiles[3 * blockIdx.x + 1], nr = tiles[3 * blockIdx.x + 2];
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1), col = lane & 31, half = lane >> 5;
+    const int n0 = (blockIdx.y * 4 + wave) * 32 * CN;
+    if (n0 >= N) return;
+    const uint16_t* ap[RM];
+#pragma unroll
+    for (int i = 0; i < RM; i++) {
+        const int r = 32 * i + col;
+        const int row = r0 + (r < nr ? r : 0);
+        const int src = a_div > 0 ? row_pair[row] / a_div : row;
+        ap[i] = a + (size_t)src * lda + half * 8;
+    }
+    const uint16_t* wp[CN];
+#pragma unroll
+    for (int j = 0; j < CN; j++) {
+        int n = n0 + 32 * j + col;
+        n = n < N ? n : N - 1;
+        wp[j] = w + ((size_t)e * N + n) * K + half * 8;
+    }
+    mfloatx16 acc[RM][CN];
+#pragma unroll
+    for (int i = 0; i < RM; i++)
+#pragma unroll
+        for (int j = 0; j < CN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+#pragma unroll 2
+    for (int k = 0; k < K; k += 16) {
+        MFrag af[RM], wf[CN];
+#pragma unroll
+        for (int i = 0; i < RM; i++) af[i].u = *reinterpret_cast<const uint4*>(ap[i] + k);
+#pragma unroll
+        for (int j = 0; j < CN; j++) wf[j].u = *reinterpret_cast<const uint4*>(wp[j] + k);
+#pragma unroll
+        for (int i = 0; i < RM; i++)
+#pragma unroll
+            for (int j = 0; j < CN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i].v, wf[j].v, acc[i][j], 0, 0, 0);
+    }
+    // element r of a lane: row 8 (r / 4) + 4 half + r % 4, column lane % 32 of its 32 x 32 block
+#pragma unroll
+    for (int i = 0; i < RM; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int row = 32 * i + 8 * (r / 4) + 4 * half + (r % 4);
+            if (row >= nr) continue;
+            const int pair = (out_by_pair || pair_scale) ? row_pair[r0 + row] : 0;
+            const float sc = pair_scale ? pair_scale[pair] : 1.f;
+            const size_t orow = out_by_pair ? (size_t)pair : (size_t)(r0 + row);
+#pragma unroll
+            for (int j = 0; j < CN; j++) {
+                const int n = n0 + 32 * j + col;
+                if (n < N) out[orow * ldo + n] = from_f32<TO>(moe_act(act, acc[i][j][r]) * sc);
+            }
+        }
+    }
+}
+
+extern "C" int hfa_moe_tile_rows(int dtype, int n_pairs, int n_experts, int N, int K) {
+    if (dtype == HFA_BF16 && K % 16 == 0 && N % 32 == 0) return n_pairs >= 48 * n_experts ? 64 : 32;
+    return PM;
+}
+
+extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const void* w, const int* row_pair,
+                            const int* tiles, const int* n_tiles, int max_tiles, int tile_rows, void* out, int ldo,
+                            int out_dtype, int out_by_pair, const float* pair_scale, int act, int N, int K,
+                            int force_plain, hipStream_t stream) {
+    HFA_REQUIRE(a && w && row_pair && tiles && n_tiles && out && max_tiles > 0 && N > 0 && K > 0 && lda >= K && ldo >= N,
+                "moe_gemm: bad arguments");
+    HFA_REQUIRE((dtype == HFA_F32 || dtype == HFA_BF16) && (out_dtype == HFA_F32 || out_dtype == HFA_BF16), "moe_gemm: unknown dtype");
+    HFA_REQUIRE(act >= 0 && act <= HFA_ACT_RELU2 && a_div >= 0, "moe_gemm: bad activation or divisor");
+    const bool mfma = !force_plain && dtype == HFA_BF16 && K % 16 == 0 && N % 32 == 0 && lda % 8 == 0 &&
+                      (tile_rows == 32 || tile_rows == 64) && ((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0;
+    if (mfma) {
+        const int cn = N % 256 == 0 && N >= 512 ? 2 : 1;
+        dim3 grid(max_tiles, (N + 128 * cn - 1) / (128 * cn));
+#define MOE_ARGS (const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles, n_tiles
+#define MOE_TAIL ldo, out_by_pair, pair_scale, act, N, K
+#define MOE_GO(RM, CN)                                                                                                  \
+    do {                                                                                                                \
+        if (out_dtype == HFA_F32) moe_gemm_mfma_kernel<RM, CN, float><<<grid, 256, 0, stream>>>(MOE_ARGS, (float*)out, MOE_TAIL); \
+        else moe_gemm_mfma_kernel<RM, CN, bf16><<<grid, 256, 0, stream>>>(MOE_ARGS, (bf16*)out, MOE_TAIL);                  \
+    } while (0)
+        if (tile_rows == 64) { if (cn == 2) MOE_GO(2, 2); else MOE_GO(2, 1); }
+        else { if (cn == 2) MOE_GO(1, 2); else MOE_GO(1, 1); }
+#undef MOE_GO
+#undef MOE_ARGS
+#undef MOE_TAIL
+    } else {
+        HFA_REQUIRE(tile_rows <= PM, "moe_gemm: the plain kernel takes tiles of at most %d rows, got %d", PM, tile_rows);
+        dim3 grid(max_tiles, (N + PN - 1) / PN);
+        if (dtype == HFA_F32 && out_dtype == HFA_F32)
+            moe_gemm_plain_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)a, lda, a_div, (const float*)w, row_pair, tiles,
+                                                                          n_tiles, (float*)out, ldo, out_by_pair, pair_scale, act, N, K);
+        else if (dtype == HFA_BF16 && out_dtype == HFA_F32)
+            moe_gemm_plain_kernel<bf16, float><<<grid, 256, 0, stream>>>((const bf16*)a, lda, a_div, (const bf16*)w, row_pair, tiles,
+                                                                         n_tiles, (float*)out, ldo, out_by_pair, pair_scale, act, N, K);
+        else if (dtype == HFA_BF16 && out_dtype == HFA_BF16)
+            moe_gemm_plain_kernel<bf16, bf16><<<grid, 256, 0, stream>>>((const bf16*)a, lda, a_div, (const bf16*)w, row_pair, tiles,
+                                                                        n_tiles, (bf16*)out, ldo, out_by_pair, pair_scale, act, N, K);
+        else
+            HFA_REQUIRE(false, "moe_gemm: fp32 operands give fp32 results");
+    }
+    HFA_LAUNCH_CHECK("moe_gemm");
+    return 0;
+}
+
+// ---- the weighted sum -----------------------------------------------------------------------
+// x[t, :] += y[t * top, :] + ... + y[t * top + top - 1, :] (fp32; the weights are in y already), choices in order.
+__global__ void moe_combine_kernel(const float* __restrict__ y, float* __restrict__ x, int top, int width, size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = i / width, c = i % width;
+        float s = 0.f;
+        for (int k = 0; k < top; k++) s += y[(t * top + k) * width + c];
+        x[i] += s;
+    }
+}
+
+extern "C" int hfa_moe_combine(const float* y, float* x, int n_tokens, int top, int width, hipStream_t stream) {
+    HFA_REQUIRE(y && x && n_tokens > 0 && top > 0 && width > 0, "moe_combine: bad arguments");
+    const size_t total = (size_t)n_tokens * width;
+    const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    moe_combine_kernel<<<blocks, 256, 0, stream>>>(y, x, top, width, total);
+    HFA_LAUNCH_CHECK("moe_combine");
+    return 0;
+}

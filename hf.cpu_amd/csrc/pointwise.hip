@@ -1,0 +1,118 @@
+// Layer norm with scale and shift, the activations of the plain feed-forward layers (erf gelu, tanh gelu,
+// squared relu) and the soft cap of the logits.
+#include "api.h"
+#include "common.h"
+
+#define LN_PLANE_BATCH 8
+
+// ---- layer norm -------------------------------------------------------------------------
+// out[r, :] = (x - mean) / sqrt(var + eps) * w + b, var = the mean squared deviation, all in fp32. One block a
+// row; mean and variance are summed in a fixed order in two passes over the row (the deviations are formed from
+// the finished mean, so a row far from zero loses nothing), and a row's result does not depend on the rest of the
+// launch. As in hfa_rmsnorm, a product that left its result as partial sums (the residual sum of the layer before)
+// is finished first: x[r, :] += sum over splits + bias, written back.
+template <typename TO>
+__global__ __launch_bounds__(1024) void layernorm_kernel(float* __restrict__ x, const float* __restrict__ w,
+                                                        const float* __restrict__ b, TO* __restrict__ out,
+                                                        const int* __restrict__ rows, int width, float eps,
+                                                        const float* __restrict__ partial, int splits,
+                                                        const float* __restrict__ pbias, int n_rows) {
+    __shared__ float red[17];
+    const int r = blockIdx.x;
+    const int xr = rows ? rows[r] : r;
+    float* src = x + (size_t)xr * width;
+    float sum = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        float v = src[i];
+        if (splits > 0) {
+            for (int s0 = 0; s0 < splits; s0 += LN_PLANE_BATCH) {
+                float p[LN_PLANE_BATCH];
+#pragma unroll
+                for (int u = 0; u < LN_PLANE_BATCH; u++)
+                    p[u] = s0 + u < splits ? partial[((size_t)(s0 + u) * n_rows + xr) * width + i] : 0.f;
+#pragma unroll
+                for (int u = 0; u < LN_PLANE_BATCH; u++) v += p[u];
+            }
+            if (pbias) v += pbias[i];
+            src[i] = v;
+        }
+        sum += v;
+    }
+    const float mean = block_sum(sum, red) / (float)width;      // the barriers inside also order the writes of x
+    float sq = 0.f;
+    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+        const float d = src[i] - mean;
+        sq = fmaf(d, d, sq);
+    }
+    const float inv = 1.0f / sqrtf(block_sum(sq, red) / (float)width + eps);
+    TO* dst = out + (size_t)r * width;
+    for (int i = threadIdx.x; i < width; i += blockDim.x)
+        dst[i] = from_f32<TO>(fmaf((src[i] - mean) * inv, w[i], b ? b[i] : 0.f));
+}
+
+extern "C" int hfa_layernorm(float* x, const float* w, const float* b, void* out, int out_dtype, const int* rows,
+                             int n_rows, int width, float eps, const float* partial, int splits,
+                             const float* partial_bias, int x_rows, hipStream_t stream) {
+    HFA_REQUIRE(x && w && out && n_rows > 0 && width > 0, "layernorm: bad arguments");
+    HFA_REQUIRE(out_dtype == HFA_F32 || out_dtype == HFA_BF16, "layernorm: unknown dtype %d", out_dtype);
+    HFA_REQUIRE(splits == 0 || (partial && !rows), "layernorm: partial sums go with all rows in order");
+    int threads = width >= 4096 ? 1024 : width >= 1024 ? 512 : width >= 256 ? 256 : 64;
+    if (out_dtype == HFA_F32)
+        layernorm_kernel<float><<<n_rows, threads, 0, stream>>>(x, w, b, (float*)out, rows, width, eps, partial, splits,
+                                                                partial_bias, x_rows);
+    else
+        layernorm_kernel<bf16><<<n_rows, threads, 0, stream>>>(x, w, b, (bf16*)out, rows, width, eps, partial, splits,
+                                                               partial_bias, x_rows);
+    HFA_LAUNCH_CHECK("layernorm");
+    return 0;
+}
+
+// ---- activations ------------------------------------------------------------------------
+__device__ __forceinline__ float act_apply(int kind, float z) {
+    if (kind == HFA_ACT_GELU_ERF) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+    if (kind == HFA_ACT_GELU_TANH) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+    if (kind == HFA_ACT_RELU2) { const float r = fmaxf(z, 0.f); return r * r; }
+    return z;
+}
+
+template <typename T>
+__global__ void activation_kernel(const T* __restrict__ in, int ldi, T* __restrict__ out, int ldo, int width, int kind,
+                                  size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / width, c = i % width;
+        out[r * ldo + c] = from_f32<T>(act_apply(kind, to_f32(in[r * ldi + c])));
+    }
+}
+
+extern "C" int hfa_activation(const void* in, int ldi, void* out, int ldo, int dtype, int n_rows, int width, int kind,
+                              hipStream_t stream) {
+    HFA_REQUIRE(in && out && n_rows > 0 && width > 0 && ldi >= width && ldo >= width, "activation: bad arguments");
+    HFA_REQUIRE(kind >= HFA_ACT_GELU_ERF && kind <= HFA_ACT_RELU2, "activation: unknown kind %d", kind);
+    HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "activation: unknown dtype %d", dtype);
+    const size_t total = (size_t)n_rows * width;
+    const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    if (dtype == HFA_F32)
+        activation_kernel<float><<<blocks, 256, 0, stream>>>((const float*)in, ldi, (float*)out, ldo, width, kind, total);
+    else
+        activation_kernel<bf16><<<blocks, 256, 0, stream>>>((const bf16*)in, ldi, (bf16*)out, ldo, width, kind, total);
+    HFA_LAUNCH_CHECK("activation");
+    return 0;
+}
+
+// ---- soft cap ---------------------------------------------------------------------------
+// x <- cap * tanh(x / cap), fp32, in place.
+__global__ void softcap_kernel(float* __restrict__ x, int ld, int width, float cap, float inv_cap, size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        float* p = x + (i / width) * ld + i % width;
+        *p = cap * tanhf(*p * inv_cap);
+    }
+}
+
+extern "C" int hfa_softcap(float* x, int ld, int n_rows, int width, float cap, hipStream_t stream) {
+    HFA_REQUIRE(x && n_rows > 0 && width > 0 && ld >= width && cap > 0.f, "softcap: bad arguments");
+    const size_t total = (size_t)n_rows * width;
+    const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    softcap_kernel<<<blocks, 256, 0, stream>>>(x, ld, width, cap, 1.0f / cap, total);
+    HFA_LAUNCH_CHECK("softcap");
+    return 0;
+}

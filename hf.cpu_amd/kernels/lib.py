@@ -21,10 +21,17 @@ _SIGNATURES = {
     "hfa_gemm_rows": [I, P, I, P, I, I, I, I, P, P, I, F, F, P, I, I, P, I, P, P, P, I, P, I, P],
     "hfa_gemm_rows_supports": [I, I, I, I, I, I],
     "hfa_rope_store": [P, I, I, P, P, I, I, I, I, I, P, P, P, I, I, P, I, P, P],
-    "hfa_paged_attention": [P, I, I, P, P, I, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, F, P, P, c_size_t, I, P],
+    "hfa_paged_attention": [P, I, I, P, P, I, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, I, F, P, P, c_size_t, I, P],
     "hfa_rope_table": [P, P, I, P, I, P],
     "hfa_decode_attention_supports": [I, I, I, I, I, I, I, I],
-    "hfa_decode_attention": [P, I, P, P, P, I, P, P, I, P, P, P, I, I, P, I, I, I, I, I, I, F, P, c_size_t, P],
+    "hfa_decode_attention": [P, I, P, P, P, I, P, P, I, P, P, P, I, I, P, I, I, I, I, I, I, I, F, P, c_size_t, P],
+    "hfa_layernorm": [P, P, P, P, I, P, I, I, F, P, I, P, I, P],
+    "hfa_activation": [P, I, P, I, I, I, I, I, P],
+    "hfa_softcap": [P, I, I, I, F, P],
+    "hfa_moe_route": [P, I, I, I, I, I, I, I, I, F, P, P, P],
+    "hfa_moe_plan": [P, I, I, I, P, P, P, P],
+    "hfa_moe_gemm": [P, I, I, I, P, P, P, P, I, I, P, I, I, I, P, I, I, I, I, P],
+    "hfa_moe_combine": [P, P, I, I, I, P],
     "hfa_swiglu": [P, P, I, I, I, P],
     "hfa_scatter_i32": [P, P, P, I, P],
     "hfa_move_i32": [P, P, P, P, I, P],
@@ -60,6 +67,8 @@ def library():
             lib.hfa_probe_mfma_threads.argtypes = []
             lib.hfa_attention_prompt_rows.restype = c_int
             lib.hfa_attention_prompt_rows.argtypes = []
+            lib.hfa_moe_tile_rows.restype = c_int
+            lib.hfa_moe_tile_rows.argtypes = [c_int] * 5
             for name, args in _SIGNATURES.items():
                 fn = getattr(lib, name)
                 fn.argtypes = args

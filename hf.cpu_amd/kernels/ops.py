@@ -400,11 +400,16 @@ class Ops:
                                              _code(p.out), _rows(p.out, "gemm out"), 1 if p.accumulate else 0, 0,
                                              M, N, self._stream()))
 
-    def gemm(self, a, w, out, bias=None, accumulate=False, defer=False, swiglu=False):
+    def gemm(self, a, w, out, bias=None, accumulate=False, defer=False, swiglu=False, activation=None):
         """out (+)= a @ w.T + bias, fp32 accumulation. ``defer``: if the kernel split K, leave the
         partial sums for the next kernel that reads ``out`` (see the module's text).
         ``swiglu``: w's rows come in blocks of 32 gate, 32 up (``interleave_gate_up``) and
-        out = silu(gate) * up has half as many columns."""
+        out = silu(gate) * up has half as many columns. ``activation``: ``out = act(a @ w.T + bias)`` (see ``activation``)."""
+        if activation is not None:
+            if accumulate or swiglu:
+                fail(EINVAL, "gemm: an activation goes with a plain output")
+            self.gemm(a, w, out, bias=bias)
+            return self.activation(activation, out, out)
         self.settle()
         lda, ldw, ldo = _rows(a, "gemm a"), _rows(w, "gemm w"), _rows(out, "gemm out")
         M, K = a.shape
@@ -515,19 +520,21 @@ class Ops:
             None if pend is None or pend.bias is None else pend.bias.data_ptr(), self._stream()))
 
     def paged_attention(self, q, n_heads, n_kv_heads, head_dim, cache, step, window, scale, out, slopes=None,
-                        v_head_dim=None):
+                        v_head_dim=None, mask_chunk=0):
         """Attention of the first ``n_heads * head_dim`` columns of ``q`` over ``cache``. ``slopes``
         (fp32, one per query head): the score of key j for the query at p gets ``slopes[h] * (j - p)``
         added, for position encodings that enter the scores; the plain kernel then runs, as it does when
-        value heads have a size of their own (``v_head_dim``; ``out`` then has that many columns a head)."""
+        value heads have a size of their own (``v_head_dim``; ``out`` then has that many columns a head).
+        ``mask_chunk`` > 0: a query sees only the keys of its own run of that many positions, counted from 0."""
         v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
+        mask_chunk = int(mask_chunk)
         self._scaled.pop(out.data_ptr(), None)               # whatever `out` held, it is no norm's lazy output any more
         lr = self._lazy_rope
         if lr is not None and lr.qkv.data_ptr() == q.data_ptr() and lr.cache is cache and slopes is None \
                 and step.max_q_len == 1 and step.n_seqs == q.shape[0] and not self.force_plain_attention \
                 and out.dtype == torch.bfloat16 and v_head_dim == head_dim and lr.args[4:7] == (n_heads, n_kv_heads, head_dim) \
                 and cache.k.numel() < 1 << 32 and cache.k.shape[0] < 1 << 24:
-            return self._decode_attention(lr, step, window, scale, out)
+            return self._decode_attention(lr, step, window, scale, out, mask_chunk)
         self.settle()
         if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != n_heads or not slopes.is_contiguous()
                                    or slopes.device != q.device):
@@ -557,7 +564,7 @@ class Ops:
                 cache.k.shape[1], cache.v.shape[1], g.block_table.data_ptr(), g.block_table.shape[1],
                 step.token_slot.data_ptr() + 4 * first, step.positions.data_ptr() + 4 * first, q_start.data_ptr(), n_seqs,
                 max_q_len, step.max_seq_len, out.data_ptr() + first * ldo * out.element_size(), ldo, n_tokens, n_heads,
-                n_kv_heads, head_dim, v_head_dim, cache.page_tokens, int(window), float(scale),
+                n_kv_heads, head_dim, v_head_dim, cache.page_tokens, int(window), mask_chunk, float(scale),
                 None if slopes is None else slopes.data_ptr(), self.attn_workspace.data_ptr(),
                 self.attn_workspace.numel(), 1 if plain else 0, self._stream()))
 
@@ -574,7 +581,7 @@ class Ops:
         else:
             call(0, T, step.q_start, step.n_seqs, step.max_q_len)
 
-    def _decode_attention(self, lr, step, window, scale, out):
+    def _decode_attention(self, lr, step, window, scale, out, mask_chunk=0):
         """Rotation, the store of the new keys and values and attention over the cache for decoded tokens, in one
         kernel: the queued ``rope_store`` (``lr``) and this call together."""
         qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map, _ = lr.args
@@ -596,7 +603,8 @@ class Ops:
             cache.v.data_ptr(), cache.k.shape[1], _ints(slot_map, "slot_map", T), g.block_table.data_ptr(),
             g.block_table.shape[1], _ints(step.token_slot, "token_slot", T), _ints(step.positions, "positions", T),
             _ints(step.q_start, "q_start", T + 1), T, step.max_seq_len, out.data_ptr(), _rows(out, "attention out"),
-            n_heads, n_kv_heads, head_dim, cache.page_tokens, int(window), float(scale), self.attn_workspace.data_ptr(),
+            n_heads, n_kv_heads, head_dim, cache.page_tokens, int(window), int(mask_chunk), float(scale),
+            self.attn_workspace.data_ptr(),
             self.attn_workspace.numel(), self._stream()))
 
     def swiglu(self, gate_up, out):
@@ -607,6 +615,102 @@ class Ops:
                 or out.dtype != gate_up.dtype or F2 % 2:
             fail(EINVAL, "swiglu: expected contiguous [T, 2F] in and [T, F] out of one dtype")
         self._check(self.lib.hfa_swiglu(gate_up.data_ptr(), out.data_ptr(), _code(out), T, F2 // 2, self._stream()))
+
+    # ---- layer norm, plain activations, soft cap -----------------------------------------------------------------
+    def layernorm(self, x, weight, bias, eps, out, rows=None):
+        """``out[r] = (x[rows[r]] - mean) / sqrt(var + eps) * weight + bias`` in fp32 (``bias`` None: no shift). A
+        deferred product into ``x`` (the residual sum before the norm) is added up by the same kernel."""
+        R, E = out.shape[0], x.shape[1]
+        if x.dtype != torch.float32 or weight.dtype != torch.float32 or not x.is_contiguous() or not out.is_contiguous() \
+                or out.shape[1] != E or weight.numel() != E or (bias is not None and (bias.dtype != torch.float32 or bias.numel() != E)):
+            fail(EINVAL, "layernorm: x, weight and bias must be fp32, contiguous, and of one width with out")
+        if rows is None and R != x.shape[0]:
+            fail(EINVAL, "layernorm: without row indices the output must have x's rows")
+        self._scaled.pop(out.data_ptr(), None)
+        pend = self._take_pending(x) if rows is None else None
+        if pend is None:
+            self.settle()
+        else:
+            self._source_changes(x)
+        self._check(self.lib.hfa_layernorm(
+            x.data_ptr(), weight.data_ptr(), None if bias is None else bias.data_ptr(), out.data_ptr(), _code(out),
+            None if rows is None else _ints(rows, "layernorm rows", R), R, E, float(eps),
+            None if pend is None else self.workspace.data_ptr(), 0 if pend is None else pend.splits,
+            None if pend is None or pend.bias is None else pend.bias.data_ptr(), x.shape[0], self._stream()))
+
+    ACTIVATIONS = {"gelu_erf": 1, "gelu_tanh": 2, "relu2": 3}
+
+    def activation(self, kind, src, out):
+        """``out = act(src)`` elementwise, computed in fp32: ``gelu_erf``, ``gelu_tanh`` or ``relu2`` (relu squared)."""
+        if kind not in self.ACTIVATIONS:
+            fail(ENOTSUP, f"activation '{kind}' is not one of {', '.join(sorted(self.ACTIVATIONS))}")
+        self.settle()
+        self._whole(src)
+        self._scaled.pop(out.data_ptr(), None)
+        if src.shape != out.shape or src.dtype != out.dtype or src.dim() != 2:
+            fail(EINVAL, "activation: input and output must be matrices of one shape and dtype")
+        self._check(self.lib.hfa_activation(src.data_ptr(), _rows(src, "activation in"), out.data_ptr(), _rows(out, "activation out"),
+                                            _code(out), src.shape[0], src.shape[1], self.ACTIVATIONS[kind], self._stream()))
+
+    def softcap(self, x, cap):
+        """``x <- cap * tanh(x / cap)`` on fp32 rows, in place."""
+        self.settle(x)
+        if x.dtype != torch.float32 or x.dim() != 2:
+            fail(EINVAL, "softcap: expected an fp32 matrix")
+        if x.shape[0]:
+            self._check(self.lib.hfa_softcap(x.data_ptr(), _rows(x, "softcap"), x.shape[0], x.shape[1], float(cap), self._stream()))
+
+    # ---- mixture of experts ------------------------------------------------------------------------------------------
+    def moe_route(self, logits, top, n_groups, keep, scoring="softmax", renorm=True, out_scale=1.0):
+        """(ids [T, top] int32, weights [T, top] fp32) from fp32 router logits [T, E]: see ``hfa_moe_route``."""
+        self.settle()
+        T, E = logits.shape
+        if logits.dtype != torch.float32 or scoring not in ("softmax", "sigmoid"):
+            fail(EINVAL, "moe_route: fp32 logits and softmax or sigmoid scoring")
+        ids = self.scratch("moe_ids", (T, top), torch.int32)
+        wts = self.scratch("moe_weights", (T, top), torch.float32)
+        self._check(self.lib.hfa_moe_route(logits.data_ptr(), _rows(logits, "router logits"), T, E, int(top), int(n_groups), int(keep),
+                                           0 if scoring == "softmax" else 1, 1 if renorm else 0, float(out_scale),
+                                           ids.data_ptr(), wts.data_ptr(), self._stream()))
+        return ids, wts
+
+    def moe_experts(self, h, ids, weights, w_up, w_down, act, x):
+        """``x[t] += sum_k weights[t, k] * w_down[ids[t, k]] act(w_up[ids[t, k]] h[t])``: ``w_up`` is [E, F, width],
+        ``w_down`` [E, width, F]. The pairs are put in expert order on the device, each expert's rows go through the
+        two products in tiles, and the weighted results are added to ``x`` (fp32) choice by choice."""
+        self.settle()
+        self._whole(h)
+        self._source_changes(x)
+        T, W = h.shape
+        E, F, _ = w_up.shape
+        top = ids.shape[1]
+        n_pairs = T * top
+        if act not in self.ACTIVATIONS:
+            fail(ENOTSUP, f"activation '{act}' is not one of {', '.join(sorted(self.ACTIVATIONS))}")
+        if tuple(w_up.shape) != (E, F, W) or tuple(w_down.shape) != (E, W, F) or not w_up.is_contiguous() or not w_down.is_contiguous() \
+                or w_up.dtype != h.dtype or w_down.dtype != h.dtype or x.dtype != torch.float32 or tuple(x.shape) != (T, W) \
+                or not x.is_contiguous() or tuple(weights.shape) != (T, top) or weights.dtype != torch.float32:
+            fail(EINVAL, "moe_experts: the experts' matrices, the activations and the residual stream do not fit")
+        code = _code(h)
+        plain = 1 if self.force_plain_gemm else 0
+        # one size of tile for both products: rows are put into tiles once
+        tile_rows = 32 if plain else min(int(self.lib.hfa_moe_tile_rows(code, n_pairs, E, F, W)),
+                                         int(self.lib.hfa_moe_tile_rows(code, n_pairs, E, W, F)))
+        max_tiles = n_pairs // tile_rows + E
+        row_pair = self.scratch("moe_row_pair", (n_pairs,), torch.int32)
+        tiles = self.scratch("moe_tiles", (3 * max_tiles + 1,), torch.int32)
+        n_tiles = tiles[3 * max_tiles:]
+        self._check(self.lib.hfa_moe_plan(_ints(ids, "moe ids", n_pairs), n_pairs, E, tile_rows, row_pair.data_ptr(), tiles.data_ptr(),
+                                          n_tiles.data_ptr(), self._stream()))
+        mid = self.scratch("moe_act", (n_pairs, F), h.dtype)
+        y = self.scratch("moe_out", (n_pairs, W), torch.float32)
+        self._check(self.lib.hfa_moe_gemm(h.data_ptr(), _rows(h, "moe h"), code, top, w_up.data_ptr(), row_pair.data_ptr(),
+                                          tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, mid.data_ptr(), F, code, 0, None,
+                                          self.ACTIVATIONS[act], F, W, plain, self._stream()))
+        self._check(self.lib.hfa_moe_gemm(mid.data_ptr(), F, code, 0, w_down.data_ptr(), row_pair.data_ptr(), tiles.data_ptr(),
+                                          n_tiles.data_ptr(), max_tiles, tile_rows, y.data_ptr(), W, F32, 1, weights.data_ptr(), 0, W, F,
+                                          plain, self._stream()))
+        self._check(self.lib.hfa_moe_combine(y.data_ptr(), x.data_ptr(), T, top, W, self._stream()))
 
     def scatter_i32(self, dst, idx, val):
         n = idx.numel()

@@ -19,7 +19,13 @@ class Attention(Part):
     values (src/model.c:499-528); ``x += Wo att`` (src/model.c:606-609).
 
     A key at ``pk`` is visible to a query at ``pq`` iff ``0 <= pq - pk`` and, when
-    ``window > 0``, ``pq - pk < window``.
+    ``window > 0``, ``pq - pk < window``, and, when ``mask_chunk > 0``, ``pq // mask_chunk == pk // mask_chunk``
+    (runs of ``mask_chunk`` positions counted from the start of the sequence, wherever a prompt was cut).
+
+    ``own_kv=False``: the mixer has no key and value projections and no cache of its own; the plan's schedule lets
+    its entry read an earlier entry's cache (``ScheduleEntry.cache_of``), with its own queries, scale and mask.
+
+    ``names`` gives the tensors' names after ``prefix`` (keys q, k, v, o, and q_bias, k_bias, v_bias, o_bias).
 
     A position encoding that enters the scores instead of the queries and keys has an
     attribute ``score_slopes`` (fp32 on the device, one per query head): the score then is
@@ -30,7 +36,7 @@ class Attention(Part):
 
 
     def __init__(self, hidden_size, n_heads, n_kv_heads, head_dim, qkv_bias, window, position,
-                 scale=None, out_bias=False, v_head_dim=None, prefix=""):
+                 scale=None, out_bias=False, v_head_dim=None, prefix="", mask_chunk=0, own_kv=True, names=None):
         """``v_head_dim``: the size of a value head where it is not ``head_dim`` (key rows of the cache are
         then ``n_kv_heads * head_dim`` wide, value rows ``n_kv_heads * v_head_dim``, and the output
         projection reads ``n_heads * v_head_dim`` columns; such a mixer runs the plain kernels)."""
@@ -44,6 +50,13 @@ class Attention(Part):
         self.qkv_bias = bool(qkv_bias)
         self.out_bias = bool(out_bias)
         self.window = int(window)
+        self.mask_chunk = int(mask_chunk)
+        self.own_kv = bool(own_kv)
+        self.names = {n: f"{n}_proj.weight" for n in "qkvo"}
+        self.names.update({f"{n}_bias": f"{n}_proj.bias" for n in "qkvo"})
+        self.names.update(names or {})
+        if self.window < 0 or self.mask_chunk < 0:
+            fail(EINVAL, "attention: a window and a masking chunk are counted in tokens, 0 for none")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # src/model.c:507
         self.position = make_part("position", position)
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
@@ -52,37 +65,43 @@ class Attention(Part):
         return [self.position]
 
     def param_specs(self):
-        p = self.prefix
-        specs = [ParamSpec(p + "q_proj.weight", (self.QD, self.E)),
-                 ParamSpec(p + "k_proj.weight", (self.KD, self.E)),
-                 ParamSpec(p + "v_proj.weight", (self.VD, self.E)),
-                 ParamSpec(p + "o_proj.weight", (self.E, self.OD))]
+        p, nm = self.prefix, self.names
+        widths = {"q": self.QD, "k": self.KD, "v": self.VD}
+        specs = [ParamSpec(p + nm[n], (widths[n], self.E)) for n in self._projections()]
+        specs.append(ParamSpec(p + nm["o"], (self.E, self.OD)))
         if self.qkv_bias:
-            specs += [ParamSpec(p + "q_proj.bias", (self.QD,), "vector"),
-                      ParamSpec(p + "k_proj.bias", (self.KD,), "vector"),
-                      ParamSpec(p + "v_proj.bias", (self.VD,), "vector")]
+            specs += [ParamSpec(p + nm[n + "_bias"], (widths[n],), "vector") for n in self._projections()]
         if self.out_bias:
-            specs.append(ParamSpec(p + "o_proj.bias", (self.E,), "vector"))
+            specs.append(ParamSpec(p + nm["o_bias"], (self.E,), "vector"))
         return specs
 
+    def _projections(self):
+        return "qkv" if self.own_kv else "q"
+
     def cache_need(self):
+        if not self.own_kv:
+            fail(EINVAL, f"attention '{self.prefix}' has no keys and values of its own: its schedule entry must read "
+                         "another entry's cache")
         return PagedKV(self.KD, self.VD, self.window)
 
     def bind(self, params, ops):
-        p = self.prefix
+        p, nm = self.prefix, self.names
         # One matrix for the three projections that share an input: rows of q, then k, then v.
-        mats = [params[p + n + "_proj.weight"] for n in "qkv"]
+        mats = [params[p + nm[n]] for n in self._projections()]
         dt = torch.float32 if any(m.dtype == torch.float32 for m in mats) else mats[0].dtype
         self.w_qkv = memory.cat([m.to(dt) for m in mats], 0, f"{p}q, k and v in one matrix")
         if self.qkv_bias:
-            self.b_qkv = memory.cat([params[p + n + "_proj.bias"] for n in "qkv"], 0, f"{p}q, k and v biases in one vector")
-        self.w_o = params[p + "o_proj.weight"]
+            self.b_qkv = memory.cat([params[p + nm[n + "_bias"]] for n in self._projections()], 0,
+                                    f"{p}q, k and v biases in one vector")
+        self.w_o = params[p + nm["o"]]
         self.short_request_rows = ops.prompt_rows     # where the attention kernels for decoded tokens and for prompt portions part
         if self.out_bias:
-            self.b_o = params[p + "o_proj.bias"]
+            self.b_o = params[p + nm["o_bias"]]
 
     def forward(self, ops, step, h, cache, x, write_cache=True):
         T = h.shape[0]
+        if write_cache and not self.own_kv:
+            fail(EINVAL, f"attention '{self.prefix}' has no keys and values to write")
         width = self.QD + self.KD + self.VD if write_cache else self.QD
         qkv = ops.scratch("qkv", (T, width), ops.act_dtype)
         # a product that split K is added up inside the next kernel (position.store, the next norm)
@@ -95,6 +114,7 @@ class Attention(Part):
         att = ops.scratch("att", (T, self.OD), ops.act_dtype)
         with ops.section("attn"):
             ops.paged_attention(qkv, self.H, self.G, self.D, cache, step, self.window, self.scale, att,
-                                slopes=getattr(self.position, "score_slopes", None), v_head_dim=self.Dv)
+                                slopes=getattr(self.position, "score_slopes", None), v_head_dim=self.Dv,
+                                mask_chunk=self.mask_chunk)
         with ops.section("wo"):
             ops.gemm(att, self.w_o, x, bias=self.b_o, accumulate=True, defer=True)

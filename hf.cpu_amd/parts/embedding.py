@@ -9,16 +9,18 @@ class Embedding(Part):
     graph_safe = True
 
 
-    def __init__(self, vocab_size, hidden_size, prefix=""):
+    def __init__(self, vocab_size, hidden_size, prefix="", weight="weight"):
+        """The table is the tensor ``prefix + weight``."""
         super().__init__(prefix)
         self.V, self.E = vocab_size, hidden_size
+        self.name = prefix + weight
         self.table = None
 
     def param_specs(self):
-        return [ParamSpec(self.prefix + "weight", (self.V, self.E))]
+        return [ParamSpec(self.name, (self.V, self.E))]
 
     def bind(self, params, ops):
-        self.table = params[self.prefix + "weight"]
+        self.table = params[self.name]
 
     def forward(self, ops, step, out_x):
         with ops.section("embed"):
@@ -29,16 +31,17 @@ class Embedding(Part):
 class LinearHead(Part):
     """``logits = W h`` in fp32, no bias (src/model.c:633-635). With ``tied`` the
     matrix is the embedding table unless the checkpoint holds one of its own, which
-    then wins (src/model.c:156-158)."""
+    then wins (src/model.c:156-158). ``softcap`` c > 0: ``logits <- c * tanh(logits / c)``."""
     graph_safe = True
     lazy_input_ok = True
 
 
-    def __init__(self, vocab_size, hidden_size, tied, tied_to="", prefix=""):
+    def __init__(self, vocab_size, hidden_size, tied, tied_to="", prefix="", softcap=None):
         super().__init__(prefix)
         self.V, self.E = vocab_size, hidden_size
         self.tied = bool(tied)
         self.tied_to = tied_to
+        self.softcap = float(softcap) if softcap else 0.0
         self.weight = None
 
     def param_specs(self):
@@ -51,3 +54,5 @@ class LinearHead(Part):
     def forward(self, ops, h, out_logits):
         with ops.section("head"):
             ops.gemm(h, self.weight, out_logits)
+            if self.softcap > 0.0:
+                ops.softcap(out_logits, self.softcap)

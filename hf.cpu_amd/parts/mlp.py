@@ -59,3 +59,36 @@ class GatedMLP(Part):
                 ops.swiglu(gu, act)
         with ops.section("down"):
             ops.gemm(act, self.w_down, x, accumulate=True, defer=True)
+
+
+@register_part("feed_forward", "mlp")
+class PlainMLP(Part):
+    """``x += Wdown act(Wup h)`` without a gate: ``activation`` is ``gelu_erf`` (0.5 z (1 + erf(z / sqrt 2))),
+    ``gelu_tanh`` or ``relu2`` (the square of relu), computed in fp32 on the product's rounded result. ``names``: the
+    two tensors' names after ``prefix`` (keys up, down)."""
+    graph_safe = True
+
+    def __init__(self, hidden_size, intermediate_size, activation="gelu_erf", prefix="", names=None):
+        super().__init__(prefix)
+        if activation not in ("gelu_erf", "gelu_tanh", "relu2"):
+            fail(ENOTSUP, f"mlp: activation '{activation}' is not implemented")
+        self.E, self.F, self.activation = hidden_size, intermediate_size, activation
+        self.names = {"up": "up_proj.weight", "down": "down_proj.weight"}
+        self.names.update(names or {})
+        self.w_up = self.w_down = None
+
+    def param_specs(self):
+        return [ParamSpec(self.prefix + self.names["up"], (self.F, self.E)),
+                ParamSpec(self.prefix + self.names["down"], (self.E, self.F))]
+
+    def bind(self, params, ops):
+        self.w_up = params[self.prefix + self.names["up"]]
+        self.w_down = params[self.prefix + self.names["down"]]
+
+    def forward(self, ops, step, h, x):
+        T = h.shape[0]
+        act = ops.scratch("ffn_act", (T, self.F), ops.act_dtype)
+        with ops.section("up"):
+            ops.gemm(h, self.w_up, act, activation=self.activation)
+        with ops.section("down"):
+            ops.gemm(act, self.w_down, x, accumulate=True, defer=True)

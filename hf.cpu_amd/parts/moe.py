@@ -1,0 +1,70 @@
+"""Mixture of experts: a router that picks a few small feed-forward layers for every token."""
+import torch
+
+from .. import memory
+from ..registry import register_part
+from ..status import EINVAL, ENOTSUP, fail
+from .base import ParamSpec, Part
+
+
+@register_part("feed_forward", "moe")
+class MixtureOfExperts(Part):
+    """``x += sum over the chosen experts e of weight_e * Wdown_e act(Wup_e h)``.
+
+    Router: logits ``z = Wrouter h`` as fp32 sums, scores ``softmax(z)`` over all experts (``scoring="sigmoid"``: the
+    logistic function of each). The experts form ``n_groups`` equal runs of neighbours; a run scores as its best
+    expert, and only experts of the ``keep_groups`` best runs can be chosen. The ``top`` best of those are chosen;
+    their weights are their scores over the sum of the chosen scores + 1e-20 (``renormalize=False``: the scores
+    themselves), times ``weight_scale``. Experts have no gate and no biases; ``activation`` as in the plain mlp.
+
+    The experts' matrices are held stacked, [experts, ff, width] and [experts, width, ff]: one launch walks all of
+    them (``Ops.moe_experts``). ``names``: the tensors' names after ``prefix`` (keys router, up, down; up and down are
+    patterns with ``{e}`` for the expert's number)."""
+    graph_safe = True
+
+    def __init__(self, hidden_size, expert_size, n_experts, top, n_groups=1, keep_groups=1, activation="relu2",
+                 scoring="softmax", renormalize=True, weight_scale=1.0, prefix="", names=None):
+        super().__init__(prefix)
+        if activation not in ("gelu_erf", "gelu_tanh", "relu2"):
+            fail(ENOTSUP, f"moe: activation '{activation}' is not implemented")
+        if scoring not in ("softmax", "sigmoid"):
+            fail(ENOTSUP, f"moe: scoring '{scoring}' is not implemented")
+        if n_experts % n_groups or not 0 < keep_groups <= n_groups:
+            fail(EINVAL, f"moe: {n_experts} experts do not form {n_groups} equal groups of which {keep_groups} are kept")
+        if not 0 < top <= keep_groups * (n_experts // n_groups):
+            fail(EINVAL, f"moe: {top} choices among the {keep_groups * (n_experts // n_groups)} experts of the kept groups")
+        self.E, self.F, self.n_experts, self.top = hidden_size, expert_size, n_experts, top
+        self.n_groups, self.keep_groups = n_groups, keep_groups
+        self.activation, self.scoring = activation, scoring
+        self.renormalize, self.weight_scale = bool(renormalize), float(weight_scale)
+        self.names = {"router": "router.weight", "up": "experts.{e}.up_proj.weight", "down": "experts.{e}.down_proj.weight"}
+        self.names.update(names or {})
+        self.w_router = self.w_up = self.w_down = None
+
+    def _name(self, key, e=None):
+        return self.prefix + (self.names[key] if e is None else self.names[key].format(e=e))
+
+    def param_specs(self):
+        specs = [ParamSpec(self._name("router"), (self.n_experts, self.E))]
+        for e in range(self.n_experts):
+            specs += [ParamSpec(self._name("up", e), (self.F, self.E)), ParamSpec(self._name("down", e), (self.E, self.F))]
+        return specs
+
+    def bind(self, params, ops):
+        self.w_router = params[self._name("router")]
+        ups = [params.pop(self._name("up", e)) for e in range(self.n_experts)]
+        downs = [params.pop(self._name("down", e)) for e in range(self.n_experts)]
+        dt = torch.float32 if any(m.dtype == torch.float32 for m in ups + downs) else ups[0].dtype
+        self.w_up = memory.cat([m.to(dt).unsqueeze(0) for m in ups], 0, f"{self.prefix}up matrices of all experts")
+        del ups
+        self.w_down = memory.cat([m.to(dt).unsqueeze(0) for m in downs], 0, f"{self.prefix}down matrices of all experts")
+
+    def forward(self, ops, step, h, x):
+        T = h.shape[0]
+        logits = ops.scratch("router_logits", (T, self.n_experts), torch.float32)
+        with ops.section("router"):
+            ops.gemm(h, self.w_router, logits)
+            ids, weights = ops.moe_route(logits, self.top, self.n_groups, self.keep_groups, self.scoring, self.renormalize,
+                                         self.weight_scale)
+        with ops.section("experts"):
+            ops.moe_experts(h, ids, weights, self.w_up, self.w_down, self.activation, x)

@@ -1,4 +1,4 @@
-"""Root-mean-square norm with a learned scale."""
+"""Norms of the residual stream: root mean square with a learned scale, and layer norm with scale and shift."""
 from ..registry import register_part
 from .base import ParamSpec, Part
 
@@ -27,3 +27,31 @@ class RMSNorm(Part):
         """``out[r] = norm(x[rows[r]])`` (``rows`` None: every row in order). ``lazy``: the caller promises that
         ``out`` is read through ``ops.gemm`` alone (a part that says ``lazy_input_ok``); see ``Ops.rmsnorm``."""
         ops.rmsnorm(x, self.weight, self.eps, out, rows, lazy=lazy)
+
+
+@register_part("norm", "layernorm")
+class LayerNorm(Part):
+    """``y = (x - mean) / sqrt(var + eps) * w + b`` over the row, ``var`` the mean of the squared deviations, in fp32.
+    ``weight`` and ``bias`` are the suffixes of the two tensors' names after ``prefix`` (``bias`` None: no shift)."""
+    graph_safe = True
+
+    def __init__(self, size, eps, weight="weight", bias="bias", prefix=""):
+        super().__init__(prefix)
+        self.size = size
+        self.eps = float(eps)
+        self.weight_name = prefix + weight
+        self.bias_name = None if bias is None else prefix + bias
+        self.weight = self.bias = None
+
+    def param_specs(self):
+        specs = [ParamSpec(self.weight_name, (self.size,), "vector", ("one_plus_normal", 0.1))]
+        if self.bias_name is not None:
+            specs.append(ParamSpec(self.bias_name, (self.size,), "vector", ("normal", 0.1)))
+        return specs
+
+    def bind(self, params, ops):
+        self.weight = params[self.weight_name]
+        self.bias = None if self.bias_name is None else params[self.bias_name]
+
+    def forward(self, ops, x, out, rows=None):
+        ops.layernorm(x, self.weight, self.bias, self.eps, out, rows)
