@@ -140,15 +140,15 @@ int hfa_softcap(float* x, int ld, int n_rows, int width, float cap, hipStream_t 
 // + 1e-20 if renorm) * out_scale. hfa_moe_plan puts the n_pairs = n_tokens * top pairs in expert order (row_pair) and
 // lists tiles of at most tile_rows rows of one expert (tiles: 3 ints a tile, room for n_pairs / tile_rows + n_experts;
 // *n_tiles on the device). hfa_moe_gemm: for every row r of the plan, out[o(r), :] = act(a[s(r), :] . w[e(r)]^T)
-// (* pair_scale[pair] if given); w is [n_experts][N][K]; s(r) = row_pair[r] / a_div if a_div > 0 else r; o(r) =
+// (* pair_scale[pair] if given); w is [n_experts][N][K] (bf16, or fp32 beside activations of either type); s(r) = row_pair[r] / a_div if a_div > 0 else r; o(r) =
 // row_pair[r] if out_by_pair else r. tile_rows must be what hfa_moe_tile_rows gave for the plan.
 // hfa_moe_combine: x[t, :] += sum_k y[t * top + k, :].
 int hfa_moe_route(const float* logits, int ld, int n_tokens, int n_experts, int top, int n_groups, int keep,
                   int scoring, int renorm, float out_scale, int* ids, float* weights, hipStream_t stream);
 int hfa_moe_plan(const int* ids, int n_pairs, int n_experts, int tile_rows, int* row_pair, int* tiles, int* n_tiles,
                  hipStream_t stream);
-int hfa_moe_tile_rows(int dtype, int n_pairs, int n_experts, int N, int K);
-int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const void* w, const int* row_pair, const int* tiles,
+int hfa_moe_tile_rows(int dtype, int w_dtype, int n_pairs, int n_experts, int N, int K);
+int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const void* w, int w_dtype, const int* row_pair, const int* tiles,
                  const int* n_tiles, int max_tiles, int tile_rows, void* out, int ldo, int out_dtype, int out_by_pair,
                  const float* pair_scale, int act, int N, int K, int force_plain, hipStream_t stream);
 int hfa_moe_combine(const float* y, float* x, int n_tokens, int top, int width, hipStream_t stream);

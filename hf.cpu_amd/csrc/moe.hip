@@ -175,9 +175,9 @@ __device__ __forceinline__ float moe_act(int act, float z) {
 #define PM 32
 #define PN 64
 #define PK 32
-template <typename T, typename TO>
+template <typename T, typename TW, typename TO>
 __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
-    const T* __restrict__ a, int lda, int a_div, const T* __restrict__ w, const int* __restrict__ row_pair,
+    const T* __restrict__ a, int lda, int a_div, const TW* __restrict__ w, const int* __restrict__ row_pair,
     const int* __restrict__ tiles, const int* __restrict__ n_tiles, TO* __restrict__ out, int ldo, int out_by_pair,
     const float* __restrict__ pair_scale, int act, int N, int K) {
     if ((int)blockIdx.x >= *n_tiles) return;
@@ -192,7 +192,7 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
         src_s[tid] = a_div > 0 ? pair / a_div : r0 + (tid < nr ? tid : 0);
     }
     __syncthreads();
-    const T* we = w + (size_t)e * N * K;
+    const TW* we = w + (size_t)e * N * K;
     const int col = tid & (PN - 1), rg = tid / PN;          // 4 row groups of 8 rows
     float acc[8];
 #pragma unroll
@@ -301,20 +301,21 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
     }
 }
 
-extern "C" int hfa_moe_tile_rows(int dtype, int n_pairs, int n_experts, int N, int K) {
-    if (dtype == HFA_BF16 && K % 16 == 0 && N % 32 == 0) return n_pairs >= 48 * n_experts ? 64 : 32;
+extern "C" int hfa_moe_tile_rows(int dtype, int w_dtype, int n_pairs, int n_experts, int N, int K) {
+    if (dtype == HFA_BF16 && w_dtype == HFA_BF16 && K % 16 == 0 && N % 32 == 0) return n_pairs >= 48 * n_experts ? 64 : 32;
     return PM;
 }
 
-extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const void* w, const int* row_pair,
+extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const void* w, int w_dtype, const int* row_pair,
                             const int* tiles, const int* n_tiles, int max_tiles, int tile_rows, void* out, int ldo,
                             int out_dtype, int out_by_pair, const float* pair_scale, int act, int N, int K,
                             int force_plain, hipStream_t stream) {
     HFA_REQUIRE(a && w && row_pair && tiles && n_tiles && out && max_tiles > 0 && N > 0 && K > 0 && lda >= K && ldo >= N,
                 "moe_gemm: bad arguments");
-    HFA_REQUIRE((dtype == HFA_F32 || dtype == HFA_BF16) && (out_dtype == HFA_F32 || out_dtype == HFA_BF16), "moe_gemm: unknown dtype");
+    HFA_REQUIRE((dtype == HFA_F32 || dtype == HFA_BF16) && (out_dtype == HFA_F32 || out_dtype == HFA_BF16) &&
+                    (w_dtype == HFA_F32 || w_dtype == HFA_BF16), "moe_gemm: unknown dtype");
     HFA_REQUIRE(act >= 0 && act <= HFA_ACT_RELU2 && a_div >= 0, "moe_gemm: bad activation or divisor");
-    const bool mfma = !force_plain && dtype == HFA_BF16 && K % 16 == 0 && N % 32 == 0 && lda % 8 == 0 &&
+    const bool mfma = !force_plain && dtype == HFA_BF16 && w_dtype == HFA_BF16 && K % 16 == 0 && N % 32 == 0 && lda % 8 == 0 &&
                       (tile_rows == 32 || tile_rows == 64) && ((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0;
     if (mfma) {
         const int cn = N % 256 == 0 && N >= 512 ? 2 : 1;
@@ -334,17 +335,17 @@ extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const 
     } else {
         HFA_REQUIRE(tile_rows <= PM, "moe_gemm: the plain kernel takes tiles of at most %d rows, got %d", PM, tile_rows);
         dim3 grid(max_tiles, (N + PN - 1) / PN);
-        if (dtype == HFA_F32 && out_dtype == HFA_F32)
-            moe_gemm_plain_kernel<float, float><<<grid, 256, 0, stream>>>((const float*)a, lda, a_div, (const float*)w, row_pair, tiles,
-                                                                          n_tiles, (float*)out, ldo, out_by_pair, pair_scale, act, N, K);
-        else if (dtype == HFA_BF16 && out_dtype == HFA_F32)
-            moe_gemm_plain_kernel<bf16, float><<<grid, 256, 0, stream>>>((const bf16*)a, lda, a_div, (const bf16*)w, row_pair, tiles,
-                                                                         n_tiles, (float*)out, ldo, out_by_pair, pair_scale, act, N, K);
-        else if (dtype == HFA_BF16 && out_dtype == HFA_BF16)
-            moe_gemm_plain_kernel<bf16, bf16><<<grid, 256, 0, stream>>>((const bf16*)a, lda, a_div, (const bf16*)w, row_pair, tiles,
-                                                                        n_tiles, (bf16*)out, ldo, out_by_pair, pair_scale, act, N, K);
+#define MOE_PLAIN(TA, TW, TO)                                                                                          \
+    moe_gemm_plain_kernel<TA, TW, TO><<<grid, 256, 0, stream>>>((const TA*)a, lda, a_div, (const TW*)w, row_pair, tiles, n_tiles, \
+                                                                  (TO*)out, ldo, out_by_pair, pair_scale, act, N, K)
+        if (dtype == HFA_F32 && w_dtype == HFA_F32 && out_dtype == HFA_F32) MOE_PLAIN(float, float, float);
+        else if (dtype == HFA_BF16 && w_dtype == HFA_BF16 && out_dtype == HFA_F32) MOE_PLAIN(bf16, bf16, float);
+        else if (dtype == HFA_BF16 && w_dtype == HFA_BF16 && out_dtype == HFA_BF16) MOE_PLAIN(bf16, bf16, bf16);
+        else if (dtype == HFA_BF16 && w_dtype == HFA_F32 && out_dtype == HFA_F32) MOE_PLAIN(bf16, float, float);
+        else if (dtype == HFA_BF16 && w_dtype == HFA_F32 && out_dtype == HFA_BF16) MOE_PLAIN(bf16, float, bf16);
         else
-            HFA_REQUIRE(false, "moe_gemm: fp32 operands give fp32 results");
+            HFA_REQUIRE(false, "moe_gemm: this mix of operand and result types is not taken (fp32 activations go with fp32 matrices and results)");
+#undef MOE_PLAIN
     }
     HFA_LAUNCH_CHECK("moe_gemm");
     return 0;

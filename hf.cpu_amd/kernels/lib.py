@@ -30,7 +30,7 @@ _SIGNATURES = {
     "hfa_softcap": [P, I, I, I, F, P],
     "hfa_moe_route": [P, I, I, I, I, I, I, I, I, F, P, P, P],
     "hfa_moe_plan": [P, I, I, I, P, P, P, P],
-    "hfa_moe_gemm": [P, I, I, I, P, P, P, P, I, I, P, I, I, I, P, I, I, I, I, P],
+    "hfa_moe_gemm": [P, I, I, I, P, I, P, P, P, I, I, P, I, I, I, P, I, I, I, I, P],
     "hfa_moe_combine": [P, P, I, I, I, P],
     "hfa_swiglu": [P, P, I, I, I, P],
     "hfa_scatter_i32": [P, P, P, I, P],
@@ -68,7 +68,7 @@ def library():
             lib.hfa_attention_prompt_rows.restype = c_int
             lib.hfa_attention_prompt_rows.argtypes = []
             lib.hfa_moe_tile_rows.restype = c_int
-            lib.hfa_moe_tile_rows.argtypes = [c_int] * 5
+            lib.hfa_moe_tile_rows.argtypes = [c_int] * 6
             for name, args in _SIGNATURES.items():
                 fn = getattr(lib, name)
                 fn.argtypes = args

@@ -688,14 +688,14 @@ class Ops:
         if act not in self.ACTIVATIONS:
             fail(ENOTSUP, f"activation '{act}' is not one of {', '.join(sorted(self.ACTIVATIONS))}")
         if tuple(w_up.shape) != (E, F, W) or tuple(w_down.shape) != (E, W, F) or not w_up.is_contiguous() or not w_down.is_contiguous() \
-                or w_up.dtype != h.dtype or w_down.dtype != h.dtype or x.dtype != torch.float32 or tuple(x.shape) != (T, W) \
+                or w_up.dtype != w_down.dtype or (w_up.dtype != h.dtype and w_up.dtype != torch.float32) or x.dtype != torch.float32 or tuple(x.shape) != (T, W) \
                 or not x.is_contiguous() or tuple(weights.shape) != (T, top) or weights.dtype != torch.float32:
             fail(EINVAL, "moe_experts: the experts' matrices, the activations and the residual stream do not fit")
-        code = _code(h)
+        code, wcode = _code(h), _code(w_up)              # matrices stored in 32-bit stay so beside bf16 activations
         plain = 1 if self.force_plain_gemm else 0
         # one size of tile for both products: rows are put into tiles once
-        tile_rows = 32 if plain else min(int(self.lib.hfa_moe_tile_rows(code, n_pairs, E, F, W)),
-                                         int(self.lib.hfa_moe_tile_rows(code, n_pairs, E, W, F)))
+        tile_rows = 32 if plain else min(int(self.lib.hfa_moe_tile_rows(code, wcode, n_pairs, E, F, W)),
+                                         int(self.lib.hfa_moe_tile_rows(code, wcode, n_pairs, E, W, F)))
         max_tiles = n_pairs // tile_rows + E
         row_pair = self.scratch("moe_row_pair", (n_pairs,), torch.int32)
         tiles = self.scratch("moe_tiles", (3 * max_tiles + 1,), torch.int32)
@@ -704,10 +704,10 @@ class Ops:
                                           n_tiles.data_ptr(), self._stream()))
         mid = self.scratch("moe_act", (n_pairs, F), h.dtype)
         y = self.scratch("moe_out", (n_pairs, W), torch.float32)
-        self._check(self.lib.hfa_moe_gemm(h.data_ptr(), _rows(h, "moe h"), code, top, w_up.data_ptr(), row_pair.data_ptr(),
+        self._check(self.lib.hfa_moe_gemm(h.data_ptr(), _rows(h, "moe h"), code, top, w_up.data_ptr(), wcode, row_pair.data_ptr(),
                                           tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, mid.data_ptr(), F, code, 0, None,
                                           self.ACTIVATIONS[act], F, W, plain, self._stream()))
-        self._check(self.lib.hfa_moe_gemm(mid.data_ptr(), F, code, 0, w_down.data_ptr(), row_pair.data_ptr(), tiles.data_ptr(),
+        self._check(self.lib.hfa_moe_gemm(mid.data_ptr(), F, code, 0, w_down.data_ptr(), wcode, row_pair.data_ptr(), tiles.data_ptr(),
                                           n_tiles.data_ptr(), max_tiles, tile_rows, y.data_ptr(), W, F32, 1, weights.data_ptr(), 0, W, F,
                                           plain, self._stream()))
         self._check(self.lib.hfa_moe_combine(y.data_ptr(), x.data_ptr(), T, top, W, self._stream()))
