@@ -1,0 +1,159 @@
+"""``bench.py --design goridra``: prefill and decode of the Goridra design at sizes that resemble a real model's layers
+(random weights), beside Qwen2 dense at equal width, heads and layer count, with every part of a step priced against
+its roofline: flops / time against the matrix cores for a prefill's parts, bytes / time against HBM for a decode
+step's. One JSON line a size."""
+import json
+import math
+import sys
+import time
+
+HBM_PEAK = 8.0e12
+MFMA_PEAK = 2.5e15
+PROMPT, PAGE = 2048, 16
+
+# width, heads, key/value heads, head size, dense ff, experts, choices, groups, kept groups, expert ff, layers, vocabulary
+SIZES = {
+    "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=8192, experts=32, top=4, groups=4, keep=2, expert_ff=1024,
+               layers=8, vocab=32000, mask=1024),
+    "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=14336, experts=64, top=8, groups=8, keep=4, expert_ff=1024,
+               layers=4, vocab=32000, mask=1024),
+}
+
+
+def goridra_shape(z):
+    """Layers in pairs: one with keys and values of its own and a dense feed-forward, one that reads them and has
+    a mixture of experts."""
+    def mixer(kv_from):
+        m = dict(heads=z["heads"], kv_heads=z["kv_heads"], dim=z["dim"], vdim=z["dim"], scale=1.0 / math.sqrt(z["dim"]),
+                 rot=dict(dims=z["dim"], base=500000.0), mask=dict(size=z["mask"]))
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return m
+    layers = []
+    for l in range(z["layers"]):
+        if l % 2 == 0:
+            layers.append(dict(type="attention", mixer=mixer(None), mlp=dict(kind="dense", ff=z["ff"])))
+        else:
+            layers.append(dict(type="attention", mixer=mixer(l - 1), mlp=dict(
+                kind="moe", expert=dict(ff=z["expert_ff"]),
+                router=dict(experts=z["experts"], top=z["top"], groups=dict(count=z["groups"], keep=z["keep"])))))
+    return dict(architecture="Goridra", vocab=z["vocab"], width=z["width"], logit_softcap=30.0, norm=dict(eps=1e-6), layers=layers)
+
+
+def qwen2_shape(z):
+    """Qwen2 dense with the same width, heads and layer count; its gated feed-forward has the dense layer's matrices'
+    worth of weights (three matrices of 2/3 the rows)."""
+    return dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", num_hidden_layers=z["layers"], hidden_size=z["width"],
+                num_attention_heads=z["heads"], num_key_value_heads=z["kv_heads"], head_dim=z["dim"],
+                intermediate_size=z["ff"] * 2 // 3 // 128 * 128, vocab_size=z["vocab"], rope_theta=500000.0, rms_norm_eps=1e-6,
+                tie_word_embeddings=True, use_sliding_window=False, max_position_embeddings=32768, hidden_act="silu")
+
+
+def part_work(design, z, T, batch, ctx):
+    """({part: flops of a prefill of T tokens}, {part: bytes of a decode step of `batch` requests at context `ctx`}),
+    all layers together, bf16."""
+    W, H, G, D, L, V = z["width"], z["heads"], z["kv_heads"], z["dim"], z["layers"], z["vocab"]
+    QD, KD = H * D, G * D
+    if design == "qwen2":
+        F = z["ff"] * 2 // 3 // 128 * 128
+        params = {"qkv": L * W * (QD + 2 * KD), "wo": L * QD * W, "gate_up": L * 2 * F * W, "down": L * F * W, "head": V * W}
+        pre = {k: 2.0 * T * v for k, v in params.items() if k != "head"}
+        pre["attn"] = L * 4.0 * D * H * T * (T + 1) / 2
+        dec = {k: 2.0 * v for k, v in params.items()}
+        dec["attn"] = batch * ctx * 2 * KD * L * 2.0
+        return pre, dec
+    own, moe = (L + 1) // 2, L // 2
+    seen = min(ctx % z["mask"] + 1, ctx)                         # keys of the current masking chunk
+    E, top, F = z["experts"], z["top"], z["expert_ff"]
+    params = {"qkv": W * (own * (QD + 2 * KD) + moe * QD), "wo": L * QD * W, "up": own * z["ff"] * W, "down": own * z["ff"] * W,
+              "router": moe * E * W, "head": V * W}
+    pre = {k: 2.0 * T * v for k, v in params.items() if k != "head"}
+    pre["experts"] = moe * T * top * 4.0 * F * W
+    chunk = z["mask"]
+    pre["attn"] = L * 4.0 * D * H * sum(min(t % chunk + 1, t + 1) for t in range(T))
+    dec = {k: 2.0 * v for k, v in params.items()}
+    touched = E * (1.0 - (1.0 - top / E) ** batch)                # experts that a step of `batch` tokens reads, evenly routed
+    dec["experts"] = moe * touched * 2 * F * W * 2.0
+    dec["attn"] = batch * seen * 2 * KD * L * 2.0                 # readers walk their source's keys again
+    return pre, dec
+
+
+def run(args):
+    import numpy as np
+    import torch
+    import hf_cpu_amd
+    import hf_cpu_amd.session as S
+    rng = np.random.default_rng(0)
+    context = args.context
+    for size in (args.sizes.split(",") if args.sizes else list(SIZES)):
+        z = SIZES[size]
+        line = {"size": size, "dims": z, "context": context, "dtype": "bf16", "data": "synthetic"}
+        for design, shape in (("goridra", goridra_shape(z)), ("qwen2", qwen2_shape(z))):
+            cfg = hf_cpu_amd.config_from_dict(shape)
+            batches = [int(b) for b in args.batches.split(",")]
+            s = S.Session(cfg, dtype="bfloat16", ctx_max=context + 64, batch=PROMPT, page_size=PAGE, max_seqs=max(batches),
+                          kv_tokens=max(batches) * (context + 64), seed=0)
+            eng, ops = s.engine, s.ops
+
+            def prompt(n=PROMPT):
+                return [int(t) for t in rng.integers(0, z["vocab"], n)]
+            out = {}
+            times = []
+            for rep in range(4):
+                p = prompt()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                ops.argmax(eng.step([("p", p, [PROMPT - 1])])).cpu()
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t0)
+                eng.release("p")
+            pre_s = sorted(times[1:])[1]
+            out["prefill_tok_per_s"] = round(PROMPT / pre_s, 1)
+            eng.profile_start()
+            for _ in range(2):
+                eng.step([("p", prompt(), [PROMPT - 1])])
+                eng.release("p")
+            book = eng.profile_stop()["prefill"]
+            pre_w, _ = part_work(design, z, PROMPT, 1, context)
+            out["prefill_parts"] = {k: {"us": round(book.get(k, 0.0) / 2 * 1e3, 1),
+                                        "frac": round(f / (book[k] / 2 * 1e-3) / MFMA_PEAK, 4)} for k, f in pre_w.items() if book.get(k)}
+            out["prefill_parts"]["other"] = {"us": round(sum(v for k, v in book.items() if k not in pre_w) / 2 * 1e3, 1)}
+            for batch in batches:
+                ids = [("d", i) for i in range(batch)]
+                for r in ids:
+                    for at in range(0, context, PROMPT):
+                        n = min(PROMPT, context - at)
+                        eng.step([(r, prompt(n), [])])
+                toks = [int(t) for t in rng.integers(0, z["vocab"], batch)]
+
+                def one():
+                    ops.argmax(eng.step([(r, [t], [0]) for r, t in zip(ids, toks)]))
+                for _ in range(6):
+                    one()
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(args.steps):
+                    one()
+                torch.cuda.synchronize()
+                dt = (time.perf_counter() - t0) / args.steps
+                _, dec_w = part_work(design, z, PROMPT, batch, context + 6 + args.steps // 2)
+                out[f"decode_b{batch}_tok_per_s"] = round(batch / dt, 1)
+                out[f"decode_b{batch}_ms"] = round(dt * 1e3, 4)
+                out[f"decode_b{batch}_hbm_frac"] = round(sum(dec_w.values()) / dt / HBM_PEAK, 4)
+                eng.profile_start()
+                for _ in range(4):
+                    one()
+                book = eng.profile_stop()["decode"]
+                out[f"decode_b{batch}_parts"] = {k: {"us": round(book.get(k, 0.0) / 4 * 1e3, 1),
+                                                     "frac": round(b / (book[k] / 4 * 1e-3) / HBM_PEAK, 4)}
+                                                 for k, b in dec_w.items() if book.get(k)}
+                out[f"decode_b{batch}_parts"]["other"] = {"us": round(sum(v for k, v in book.items() if k not in dec_w) / 4 * 1e3, 1)}
+                for r in ids:
+                    eng.release(r)
+            line[design] = out
+            print(f"[bench] {size} {design}: prefill {out['prefill_tok_per_s']} tok/s, decode "
+                  + ", ".join(f"b{b} {out[f'decode_b{b}_tok_per_s']} tok/s" for b in batches), file=sys.stderr, flush=True)
+            del s, eng, ops
+            torch.cuda.empty_cache()
+        print(json.dumps(line), flush=True)
+    return 0

@@ -28,6 +28,9 @@ int hfa_rmsnorm(float* x, const float* w, void* out, int out_dtype, const int* r
 // `workspace` for small M); everything else, and everything when `force_plain`, runs the plain
 // fp32 multiply-add kernel. `epilogue` 1 (matrix cores only): the columns of w come in blocks of
 // 32 gate rows, 32 up rows, and out[m, f] = silu(gate) * up has N / 2 columns (src/model.c:537).
+// `epilogue` 1 + k (k = HFA_ACT_GELU_ERF, HFA_ACT_GELU_TANH or HFA_ACT_RELU2; not with `accumulate`, never deferred):
+// out[m, n] = act_k(sum + bias[n]), the activation computed in fp32 in the product's last lines (on the plain path by
+// the elementwise kernel after it).
 // `defer`: if K was split, leave the partial sums ([splits][M][N] fp32 at the start of the
 // workspace) for the caller's next kernel and report the number of splits in *pending_splits.
 // (src/model.c:408-424)
@@ -40,7 +43,7 @@ int hfa_gemm_finish(const void* partial, int splits, const float* bias, void* ou
 
 // The product for up to 32 rows in which every block owns a range of outputs and finishes them itself (bf16
 // operands, K a multiple of 128; see gemm_rows.hip), with what follows a product in a decode step in its last lines:
-//   HFA_ROWS_OUT     out[m, n] = r[m] * sum + bias[n], fp32 or bf16 (out_dtype)
+//   HFA_ROWS_OUT     out[m, n] = act(r[m] * sum + bias[n]), fp32 or bf16 (out_dtype); act = out_act (HFA_ACT_*, 0: none)
 //   HFA_ROWS_RESID   x[m, n] += sum + bias[n] (fp32, in place); ssq_out[b][m] = block b's share of sum_n x[m, n]^2
 //                    ([hfa_gemm_rows_parts()][16] floats, [..][32] from 17 rows up: give room for 32); xg[m, n] = bf16(x[m, n] * g[n]) if xg is given
 //   HFA_ROWS_SWIGLU  act[m, f] = bf16(silu(r[m] * sum_gate) * (r[m] * sum_up)), N features, w's 2 N rows in blocks of
@@ -56,7 +59,7 @@ int hfa_gemm_rows_parts(void);
 int hfa_gemm_rows_supports(int mode, int M, int N, int K, int lda, int ldw);
 int hfa_gemm_rows(int mode, const void* a, int lda, const void* w, int ldw, int M, int N, int K, const float* bias,
                   const float* ssq_in, int parts_in, float inv_width, float eps, void* out, int ldo, int out_dtype,
-                  float* x, int ldx, float* ssq_out, const float* g, void* xg, int ldxg, void* act, int ldact,
+                  int out_act, float* x, int ldx, float* ssq_out, const float* g, void* xg, int ldxg, void* act, int ldact,
                   hipStream_t stream);
 
 // Rotary position encoding on the q (and k) heads inside qkv rows [q | k | v], split-half
@@ -124,10 +127,12 @@ int hfa_layernorm(float* x, const float* w, const float* b, void* out, int out_d
 
 // out[r, c] = act(in[r, c]) for rows of `width` values with strides ldi and ldo, computed in fp32:
 // the exact gelu 0.5 z (1 + erf(z / sqrt 2)), its tanh form, or relu(z)^2.
+#ifndef HFA_ACT_GELU_ERF
 #define HFA_ACT_NONE 0
 #define HFA_ACT_GELU_ERF 1
 #define HFA_ACT_GELU_TANH 2
 #define HFA_ACT_RELU2 3
+#endif
 int hfa_activation(const void* in, int ldi, void* out, int ldo, int dtype, int n_rows, int width, int kind,
                    hipStream_t stream);
 

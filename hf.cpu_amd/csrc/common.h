@@ -68,6 +68,20 @@ __device__ __forceinline__ float block_max(float v, float* red) {
     return red[16];
 }
 
+// ---- activations of the plain feed-forward layers, computed in fp32 (kinds as in api.h) ----
+#ifndef HFA_ACT_GELU_ERF
+#define HFA_ACT_NONE 0
+#define HFA_ACT_GELU_ERF 1
+#define HFA_ACT_GELU_TANH 2
+#define HFA_ACT_RELU2 3
+#endif
+__device__ __forceinline__ float hfa_act_apply(int kind, float z) {
+    if (kind == HFA_ACT_GELU_ERF) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
+    if (kind == HFA_ACT_GELU_TANH) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
+    if (kind == HFA_ACT_RELU2) { const float r = fmaxf(z, 0.f); return r * r; }
+    return z;
+}
+
 // ---- error reporting of the launchers ---------------------------------------------------
 // Every extern "C" launcher returns 0, or a non-zero code after leaving a message that
 // hfa_last_error() returns. Bad shapes are refused before anything is launched.

@@ -14,18 +14,26 @@ extern "C" int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int 
                     (out_dtype == HFA_F32 || out_dtype == HFA_BF16),
                 "gemm: unknown dtype (a=%d w=%d out=%d)", a_dtype, w_dtype, out_dtype);
     HFA_REQUIRE(!accumulate || out_dtype == HFA_F32, "gemm: accumulation needs an fp32 output");
-    HFA_REQUIRE(epilogue == 0 || epilogue == 1, "gemm: unknown epilogue %d", epilogue);
+    HFA_REQUIRE(epilogue >= 0 && epilogue <= 1 + HFA_ACT_RELU2, "gemm: unknown epilogue %d", epilogue);
+    const int act = epilogue >= 2 ? epilogue - 1 : 0;
+    HFA_REQUIRE(!act || !accumulate, "gemm: an activation goes with a plain output, not with accumulation");
+    if (act) {
+        epilogue = 0;
+        defer = 0;
+    }
     if (pending_splits) *pending_splits = 0;
-    GemmArgs g = {a, a_dtype, lda, w, w_dtype, ldw, bias, out, out_dtype, ldo, accumulate, epilogue, M, N, K, stream};
+    GemmArgs g = {a, a_dtype, lda, w, w_dtype, ldw, bias, out, out_dtype, ldo, accumulate, epilogue, M, N, K, stream, act};
     if (!force_plain && gemm_mfma_supports(g)) return gemm_mfma_launch(g, workspace, workspace_bytes, defer, pending_splits);
     HFA_REQUIRE(epilogue == 0, "gemm: the gate/up epilogue exists only on the matrix-core path");
-    return gemm_generic_launch(g);
+    const int rc = gemm_generic_launch(g);
+    if (rc || !act) return rc;
+    return hfa_activation(out, ldo, out, ldo, out_dtype, M, N, act, stream);
 }
 
 // Finishes a product that hfa_gemm left as partial sums: out (+)= sum over splits + bias.
 extern "C" int hfa_gemm_finish(const void* partial, int splits, const float* bias, void* out, int out_dtype, int ldo,
                                int accumulate, int epilogue, int M, int N, hipStream_t stream) {
     HFA_REQUIRE(splits > 0 && M > 0 && N > 0, "gemm_finish: bad sizes");
-    GemmArgs g = {nullptr, HFA_BF16, 0, nullptr, HFA_BF16, 0, bias, out, out_dtype, ldo, accumulate, epilogue, M, N, 0, stream};
+    GemmArgs g = {nullptr, HFA_BF16, 0, nullptr, HFA_BF16, 0, bias, out, out_dtype, ldo, accumulate, epilogue, M, N, 0, stream, 0};
     return gemm_finish_launch((const float*)partial, splits, bias, out, gemm_mode_of(g), ldo, M, N, stream);
 }

@@ -12,6 +12,7 @@ struct GemmArgs {
     int epilogue;            // 0: none; 1: columns are 32 gate, 32 up, ...: out[m, f] = silu(gate) * up
     int M, N, K;
     hipStream_t stream;
+    int act;                 // HFA_ACT_* applied to a plain output (not with accumulate), 0: none
 };
 
 // Any dtype mix, any size: fp32 multiply-add over K in ascending order for every output.
@@ -37,4 +38,4 @@ int gemm_stream_launch(const GemmArgs& g, void* workspace, int slots);
 int gemm_wave_slots(const GemmArgs& g, size_t workspace_bytes);
 int gemm_wave_launch(const GemmArgs& g, void* workspace, int slots);
 int gemm_finish_launch(const float* partial, int splits, const float* bias, void* out, int mode, int ldo, int M,
-                       int N, hipStream_t stream);
+                       int N, hipStream_t stream, int act = 0);

@@ -63,7 +63,7 @@ struct MfmaCfg {
 template <class C, int MODE>
 __device__ __forceinline__ void gemm_epilogue(floatx16 (&acc)[C::FM][C::FN], const float* __restrict__ bias,
                                               void* __restrict__ out, int ldo, int M, int N, int m0, int n0, int wm,
-                                              int wn, int lane) {
+                                              int wn, int lane, int act = 0) {
     if (MODE == OUT_SWIGLU) {
         static_assert(MODE != OUT_SWIGLU || C::FN % 2 == 0, "gate and up blocks must meet in one wave");
 #pragma unroll
@@ -95,7 +95,8 @@ __device__ __forceinline__ void gemm_epilogue(floatx16 (&acc)[C::FM][C::FN], con
             for (int r = 0; r < 16; r++) {
                 const int row = m0 + wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
                 if (row >= M) continue;
-                const float v = acc[i][j][r] + b;
+                float v = acc[i][j][r] + b;
+                if ((MODE == OUT_BF16 || MODE == OUT_F32) && act) v = hfa_act_apply(act, v);
                 if (MODE == OUT_BF16) {
                     reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + col] = bf16_bits(v);
                 } else if (MODE == OUT_F32) {
@@ -126,7 +127,7 @@ struct DmaOut {
 template <class C, int BM, int BN, int MODE>
 __device__ __forceinline__ void gemm_epilogue_rows(floatx16 (&acc)[C::FM][C::FN], const float* __restrict__ bias,
                                                    void* __restrict__ out, int ldo, int M, int N, int m0, int n0,
-                                                   int wm, int wn, int lane, int tid, uint16_t* smem) {
+                                                   int wm, int wn, int lane, int tid, uint16_t* smem, int act = 0) {
     using O = DmaOut<BN, MODE>;
     static_assert(MODE != OUT_SWIGLU || C::FN % 2 == 0, "gate and up blocks must meet in one wave");
     __syncthreads();
@@ -142,6 +143,7 @@ __device__ __forceinline__ void gemm_epilogue_rows(floatx16 (&acc)[C::FM][C::FN]
                 const int row = wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
                 float v = acc[i][j][r] + b;
                 if constexpr (MODE == OUT_SWIGLU) v = (v / (1.0f + expf(-v))) * acc[i][j + 1][r];
+                else if (act) v = hfa_act_apply(act, v);
                 smem[row * O::STRIDE + col] = bf16_bits(v);
             }
         }
@@ -161,7 +163,7 @@ template <int BM, int BN, int BK, int WM, int WN, int MODE, int PF>
 __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
     const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, int ldw,
     const float* __restrict__ bias, void* __restrict__ out, int ldo, int M, int N, int K, int k_per_split,
-    int tiles_m, int tiles_n, int rows_out) {
+    int tiles_m, int tiles_n, int rows_out, int act) {
     using C = MfmaCfg<BM, BN, BK, WM, WN>;
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), wave = tid / WAVE;
@@ -276,11 +278,11 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
     if constexpr (MODE == OUT_BF16 || MODE == OUT_SWIGLU) {
         static_assert(DmaOut<BN, MODE>::bytes(BM) <= C::SMEM, "the tile of results fits the operand stages");
         if (rows_out) {                                      // uniform: the output allows 16-byte stores
-            gemm_epilogue_rows<C, BM, BN, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane, tid, smem);
+            gemm_epilogue_rows<C, BM, BN, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane, tid, smem, act);
             return;
         }
     }
-    gemm_epilogue<C, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane);
+    gemm_epilogue<C, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane, act);
 }
 
 // ---- large M (prompts): operand tiles travel global -> LDS without passing through registers ----
@@ -326,7 +328,7 @@ template <int BM, int BN, int BK, int WM, int WN, int STAGES, int MODE>
 __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
     const uint16_t* __restrict__ A, int lda, const uint16_t* __restrict__ W, int ldw,
     const float* __restrict__ bias, void* __restrict__ out, int ldo, int M, int N, int K, int k_per_split,
-    int tiles_m, int tiles_n) {
+    int tiles_m, int tiles_n, int act) {
     using C = DmaCfg<BM, BN, BK, WM, WN>;
     static_assert(STAGES >= 3, "one tile in use, the next one landed, one arriving");
     extern __shared__ __attribute__((aligned(1024))) uint16_t smem[];
@@ -459,22 +461,23 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
     for (; t + AHEAD < nk; t++) step(t, std::true_type());
     for (; t < nk; t++) step(t, std::false_type());
     if constexpr (MODE == OUT_BF16 || MODE == OUT_SWIGLU) {
-        gemm_epilogue_rows<C, BM, BN, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane, tid, smem);
+        gemm_epilogue_rows<C, BM, BN, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane, tid, smem, act);
     } else {
-        gemm_epilogue<C, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane);
+        gemm_epilogue<C, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane, act);
     }
 }
 
 // Sum of the K splits in ascending order, then bias and the output mode.
 template <int MODE>
 __global__ void gemm_finish_kernel(const float* __restrict__ partial, int splits, const float* __restrict__ bias,
-                                   void* __restrict__ out, int ldo, int M, int N) {
+                                   void* __restrict__ out, int ldo, int M, int N, int act) {
     const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= (size_t)M * N) return;
     const int row = (int)(idx / N), col = (int)(idx % N);
     float v = 0.f;
     for (int s = 0; s < splits; s++) v += partial[(size_t)s * M * N + idx];
     if (bias) v += bias[col];
+    if ((MODE == OUT_BF16 || MODE == OUT_F32) && act) v = hfa_act_apply(act, v);
     if (MODE == OUT_SWIGLU) {                 // this thread holds a gate column; its up column is 32 further
         if ((col & 32) != 0) return;
         float up = 0.f;
@@ -538,7 +541,7 @@ static int launch_cfg(const GemmArgs& g, void* out, int splits, int k_per_split)
     const int n_out = MODE == OUT_SWIGLU ? g.N / 2 : g.N;
     const int rows_out = (MODE == OUT_BF16 || MODE == OUT_SWIGLU) && g.ldo % 8 == 0 && n_out % 8 == 0 && ((uintptr_t)out & 15) == 0;
     kernel<<<grid, C::NT, C::SMEM, g.stream>>>((const uint16_t*)g.a, g.lda, (const uint16_t*)g.w, g.ldw, g.bias, out,
-                                              g.ldo, g.M, g.N, g.K, k_per_split, tiles_m, tiles_n, rows_out);
+                                              g.ldo, g.M, g.N, g.K, k_per_split, tiles_m, tiles_n, rows_out, g.act);
     HFA_LAUNCH_CHECK("gemm_mfma");
     return 0;
 }
@@ -560,7 +563,7 @@ static int launch_dma_cfg(const GemmArgs& g, void* out, int splits, int k_per_sp
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     kernel<<<dim3(tiles_m * tiles_n, 1, splits), C::NT, SMEM, g.stream>>>(
         (const uint16_t*)g.a, g.lda, (const uint16_t*)g.w, g.ldw, g.bias, out, g.ldo, g.M, g.N, g.K, k_per_split, tiles_m,
-        tiles_n);
+        tiles_n, g.act);
     HFA_LAUNCH_CHECK("gemm_dma");
     return 0;
 }
@@ -599,19 +602,19 @@ bool gemm_mfma_supports(const GemmArgs& g) {
 }
 
 int gemm_finish_launch(const float* partial, int splits, const float* bias, void* out, int mode, int ldo, int M,
-                       int N, hipStream_t stream) {
+                       int N, hipStream_t stream, int act) {
     const size_t total = (size_t)M * N;
     const int blocks = (int)((total + 255) / 256);
     if (mode == OUT_BF16)
-        gemm_finish_kernel<OUT_BF16><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N);
+        gemm_finish_kernel<OUT_BF16><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N, act);
     else if (mode == OUT_F32)
-        gemm_finish_kernel<OUT_F32><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N);
+        gemm_finish_kernel<OUT_F32><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N, act);
     else if (mode == OUT_SWIGLU && !bias && N % 64 == 0 && ldo % 4 == 0 && ((uintptr_t)out & 7) == 0 && ((uintptr_t)partial & 15) == 0)
         gemm_finish_swiglu4_kernel<<<(int)((total / 8 + 255) / 256), 256, 0, stream>>>(partial, splits, (uint16_t*)out, ldo, M, N);
     else if (mode == OUT_SWIGLU)
-        gemm_finish_kernel<OUT_SWIGLU><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N);
+        gemm_finish_kernel<OUT_SWIGLU><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N, act);
     else
-        gemm_finish_kernel<OUT_ACC><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N);
+        gemm_finish_kernel<OUT_ACC><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N, act);
     HFA_LAUNCH_CHECK("gemm_finish");
     return 0;
 }
@@ -637,7 +640,7 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
                 *pending_splits = slots;
                 return 0;
             }
-            return gemm_finish_launch((const float*)workspace, slots, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream);
+            return gemm_finish_launch((const float*)workspace, slots, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream, g.act);
         }
     }
     if (g.M <= 128) {
@@ -649,7 +652,7 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
                 *pending_splits = slots;
                 return 0;
             }
-            return gemm_finish_launch((const float*)workspace, slots, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream);
+            return gemm_finish_launch((const float*)workspace, slots, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream, g.act);
         }
     }
     const int BK = 64;
@@ -742,7 +745,7 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
             *pending_splits = parts;
             return 0;
         }
-        return gemm_finish_launch((const float*)workspace, parts, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream);
+        return gemm_finish_launch((const float*)workspace, parts, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream, g.act);
     } else if (dma_ok && 2 * tiles256 >= 128)
         rc = launch_dma<256, 128, 32, 4, 2, 6>(g, kmode, kout, 1, g.K);
     else if (BM == 128)                        // eight waves a block in both: about 2 % quicker than four with twice the accumulators
@@ -760,5 +763,5 @@ int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes,
         *pending_splits = splits;
         return 0;
     }
-    return gemm_finish_launch((const float*)workspace, splits, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream);
+    return gemm_finish_launch((const float*)workspace, splits, g.bias, g.out, mode, g.ldo, g.M, g.N, g.stream, g.act);
 }

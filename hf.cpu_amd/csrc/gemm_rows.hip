@@ -49,6 +49,7 @@ struct RowGemm {
     const float* ssq_in; int parts_in;     // [parts_in][16 or 32] shares of the sums of squares of the normed rows (32 from 17 rows up), or null
     float inv_width, eps;                  // r[m] = rsqrt(sum * inv_width + eps)
     void* out; int ldo; int out_bf16;      // OUT
+    int out_act;                           // OUT: HFA_ACT_* applied to the result, 0: none
     float* x; int ldx; float* ssq_out;     // RESID: residual stream; [gridDim.x][16 or 32] shares of the sums of squares
     const float* g; uint16_t* xg; int ldxg;   // RESID: the next norm's weight and x * g in bf16 (or null)
     uint16_t* act; int ldact;              // SWIGLU
@@ -331,7 +332,8 @@ __global__ __launch_bounds__(RG_WAVES * WAVE) void gemm_rows_kernel(const RowGem
             for (int i = tid; i < nt * 16 * MR; i += RG_WAVES * WAVE) {
                 const int tt = i / (16 * MR), m = (i >> 4) % MR, n = i & 15, col = own0 + 16 * (tg0 + tt) + n;
                 if (m < p.T && col < own1) {
-                    const float v = r_s[m] * total(tt, m, n) + (!p.bias ? 0.f : (tg0 == 0 && i == tid) ? early_b : p.bias[col]);
+                    float v = r_s[m] * total(tt, m, n) + (!p.bias ? 0.f : (tg0 == 0 && i == tid) ? early_b : p.bias[col]);
+                    if (p.out_act) v = hfa_act_apply(p.out_act, v);
                     if (p.out_bf16) reinterpret_cast<uint16_t*>(p.out)[(size_t)m * p.ldo + col] = rg_bf16(v);
                     else reinterpret_cast<float*>(p.out)[(size_t)m * p.ldo + col] = v;
                 }
@@ -447,7 +449,7 @@ extern "C" int hfa_gemm_rows_supports(int mode, int M, int N, int K, int lda, in
 
 extern "C" int hfa_gemm_rows(int mode, const void* a, int lda, const void* w, int ldw, int M, int N, int K,
                              const float* bias, const float* ssq_in, int parts_in, float inv_width, float eps,
-                             void* out, int ldo, int out_dtype, float* x, int ldx, float* ssq_out, const float* g,
+                             void* out, int ldo, int out_dtype, int out_act, float* x, int ldx, float* ssq_out, const float* g,
                              void* xg, int ldxg, void* act, int ldact, hipStream_t stream) {
     HFA_REQUIRE(mode == HFA_ROWS_OUT || mode == HFA_ROWS_RESID || mode == HFA_ROWS_SWIGLU, "gemm_rows: unknown mode %d", mode);
     HFA_REQUIRE(hfa_gemm_rows_supports(mode, M, N, K, lda, ldw),
@@ -461,7 +463,8 @@ extern "C" int hfa_gemm_rows(int mode, const void* a, int lda, const void* w, in
     p.bias = bias; p.ssq_in = ssq_in; p.parts_in = parts_in; p.inv_width = inv_width; p.eps = eps;
     if (mode == HFA_ROWS_OUT) {
         HFA_REQUIRE(out && ldo >= N && (out_dtype == HFA_F32 || out_dtype == HFA_BF16), "gemm_rows: no output, or its rows are shorter than N");
-        p.out = out; p.ldo = ldo; p.out_bf16 = out_dtype == HFA_BF16;
+        HFA_REQUIRE(out_act >= 0 && out_act <= HFA_ACT_RELU2, "gemm_rows: unknown activation %d", out_act);
+        p.out = out; p.ldo = ldo; p.out_bf16 = out_dtype == HFA_BF16; p.out_act = out_act;
         return rows_dispatch<HFA_ROWS_OUT>(p, stream);
     }
     if (mode == HFA_ROWS_RESID) {

@@ -163,13 +163,6 @@ extern "C" int hfa_moe_plan(const int* ids, int n_pairs, int n_experts, int tile
 }
 
 // ---- the experts' products ----------------------------------------------------------------
-__device__ __forceinline__ float moe_act(int act, float z) {
-    if (act == HFA_ACT_RELU2) { const float r = fmaxf(z, 0.f); return r * r; }
-    if (act == HFA_ACT_GELU_ERF) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
-    if (act == HFA_ACT_GELU_TANH) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
-    return z;
-}
-
 // Plain form, any dtype and shape: a tile of up to 32 rows x 64 columns a block, operands staged through LDS 32 k at a
 // time, every output summed over k in ascending order by one thread.
 #define PM 32
@@ -220,7 +213,7 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
     for (int i = 0; i < 8; i++) {
         const int r = rg * 8 + i;
         if (r >= nr) continue;
-        float v = moe_act(act, acc[i]);
+        float v = hfa_act_apply(act, acc[i]);
         if (pair_scale) v *= pair_scale[pair_s[r]];
         const size_t orow = out_by_pair ? (size_t)pair_s[r] : (size_t)(r0 + r);
         out[orow * ldo + n0 + col] = from_f32<TO>(v);
@@ -237,6 +230,60 @@ union MFrag {
     uint4 u;
     mbf16x8 v;
 };
+
+// Few rows an expert (decoded tokens): the experts' matrices are streamed once and that stream is the bound, so the
+// work is cut small: a block owns 32 rows x 32 columns of one expert, its four waves take a quarter of K each (K a
+// multiple of 64) with the loads of four steps on their way at a time, and the four partial tiles are added in LDS in
+// wave order.
+template <typename TO>
+__global__ __launch_bounds__(256) void moe_gemm_split_kernel(
+    const uint16_t* __restrict__ a, int lda, int a_div, const uint16_t* __restrict__ w, const int* __restrict__ row_pair,
+    const int* __restrict__ tiles, const int* __restrict__ n_tiles, TO* __restrict__ out, int ldo, int out_by_pair,
+    const float* __restrict__ pair_scale, int act, int N, int K) {
+    if ((int)blockIdx.x >= *n_tiles) return;
+    __shared__ float part_s[4][32 * 33];
+    const int e = tiles[3 * blockIdx.x], r0 = tiles[3 * blockIdx.x + 1], nr = tiles[3 * blockIdx.x + 2];
+    const int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1), col = lane & 31, half = lane >> 5;
+    const int n0 = blockIdx.y * 32;
+    const int row = r0 + (col < nr ? col : 0);
+    const int src = a_div > 0 ? row_pair[row] / a_div : row;
+    const int kq = K / 4, k0 = wave * kq;
+    const uint16_t* ap = a + (size_t)src * lda + k0 + half * 8;
+    int n = n0 + col;
+    n = n < N ? n : N - 1;
+    const uint16_t* wp = w + ((size_t)e * N + n) * K + k0 + half * 8;
+    mfloatx16 acc;
+#pragma unroll
+    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    int k = 0;
+    for (; k + 64 <= kq; k += 64) {
+        MFrag af[4], wf[4];
+#pragma unroll
+        for (int u = 0; u < 4; u++) {
+            wf[u].u = *reinterpret_cast<const uint4*>(wp + k + 16 * u);
+            af[u].u = *reinterpret_cast<const uint4*>(ap + k + 16 * u);
+        }
+#pragma unroll
+        for (int u = 0; u < 4; u++) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[u].v, wf[u].v, acc, 0, 0, 0);
+    }
+    for (; k < kq; k += 16) {
+        MFrag af, wf;
+        wf.u = *reinterpret_cast<const uint4*>(wp + k);
+        af.u = *reinterpret_cast<const uint4*>(ap + k);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af.v, wf.v, acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 16; r++) part_s[wave][(8 * (r / 4) + 4 * half + (r % 4)) * 33 + col] = acc[r];
+    __syncthreads();
+    for (int i = threadIdx.x; i < 32 * 32; i += 256) {
+        const int r = i >> 5, c = i & 31;
+        if (r >= nr || n0 + c >= N) continue;
+        const float v = ((part_s[0][r * 33 + c] + part_s[1][r * 33 + c]) + part_s[2][r * 33 + c]) + part_s[3][r * 33 + c];
+        const int pair = (out_by_pair || pair_scale) ? row_pair[r0 + r] : 0;
+        const size_t orow = out_by_pair ? (size_t)pair : (size_t)(r0 + r);
+        out[orow * ldo + n0 + c] = from_f32<TO>(hfa_act_apply(act, v) * (pair_scale ? pair_scale[pair] : 1.f));
+    }
+}
 
 template <int RM, int CN, typename TO>
 __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
@@ -295,14 +342,141 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
 #pragma unroll
             for (int j = 0; j < CN; j++) {
                 const int n = n0 + 32 * j + col;
-                if (n < N) out[orow * ldo + n] = from_f32<TO>(moe_act(act, acc[i][j][r]) * sc);
+                if (n < N) out[orow * ldo + n] = from_f32<TO>(hfa_act_apply(act, acc[i][j][r]) * sc);
+            }
+        }
+    }
+}
+
+// Matrix-core form for many rows an expert (prompt portions): a block of 2 x 2 waves owns BM rows of one expert x BN
+// columns and walks K in steps of BK through two LDS stages, as gemm_mfma_kernel does for one matrix: the next tile
+// travels global -> registers while the current one is multiplied out of LDS, then registers -> LDS, one barrier a
+// step; LDS rows are padded by 8 elements so that the 16-byte fragment reads do not conflict. The rows of `a` are
+// gathered through row_pair (their source rows wait in LDS), so every operand element is read from memory once a
+// block instead of once a wave.
+template <int BM, int BN, int BK, typename TO>
+__global__ __launch_bounds__(256) void moe_gemm_lds_kernel(
+    const uint16_t* __restrict__ a, int lda, int a_div, const uint16_t* __restrict__ w, const int* __restrict__ row_pair,
+    const int* __restrict__ tiles, const int* __restrict__ n_tiles, TO* __restrict__ out, int ldo, int out_by_pair,
+    const float* __restrict__ pair_scale, int act, int N, int K) {
+    constexpr int STRIDE = BK + 8, NT = 256, CPR = BK / 8, A_CH = BM * CPR / NT, W_CH = BN * CPR / NT;
+    constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32, STAGE = (BM + BN) * STRIDE;
+    static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0 && TM % 32 == 0 && TN % 32 == 0, "tiles spread evenly");
+    if ((int)blockIdx.x >= *n_tiles) return;
+    extern __shared__ __attribute__((aligned(16))) uint16_t smem[];       // two stages of (BM + BN) x STRIDE elements
+    __shared__ int src_s[BM], pair_s[BM];
+    const int e = tiles[3 * blockIdx.x], r0 = tiles[3 * blockIdx.x + 1], nr = tiles[3 * blockIdx.x + 2];
+    const int n0 = blockIdx.y * BN, tid = threadIdx.x, wave = tid / WAVE, lane = tid & (WAVE - 1);
+    const int wm = wave >> 1, wn = wave & 1;
+    for (int i = tid; i < BM; i += NT) {
+        const int row = r0 + (i < nr ? i : 0);
+        const int pair = row_pair[row];
+        pair_s[i] = pair;
+        src_s[i] = a_div > 0 ? pair / a_div : row;
+    }
+    __syncthreads();
+    const uint16_t* we = w + (size_t)e * N * K;
+    mfloatx16 acc[FM][FN];
+#pragma unroll
+    for (int i = 0; i < FM; i++)
+#pragma unroll
+        for (int j = 0; j < FN; j++)
+#pragma unroll
+            for (int r = 0; r < 16; r++) acc[i][j][r] = 0.f;
+    // PF register sets of loads are on their way while a tile is multiplied: a tile's trip from memory takes longer
+    // than the multiplication of one tile, and a block has nothing else to do meanwhile.
+    constexpr int PF = 3;
+    uint4 ra[PF][A_CH], rw[PF][W_CH];
+    size_t arow[A_CH];
+#pragma unroll
+    for (int i = 0; i < A_CH; i++) arow[i] = (size_t)src_s[(tid + i * NT) / CPR] * lda;
+    auto gload = [&](uint4* ra, uint4* rw, int k0) {
+#pragma unroll
+        for (int i = 0; i < A_CH; i++) {
+            const int c = tid + i * NT, kk = k0 + (c % CPR) * 8;
+            ra[i] = kk < K ? *reinterpret_cast<const uint4*>(a + arow[i] + kk) : make_uint4(0, 0, 0, 0);
+        }
+#pragma unroll
+        for (int i = 0; i < W_CH; i++) {
+            const int c = tid + i * NT, row = c / CPR, kk = k0 + (c % CPR) * 8;
+            int n = n0 + row;
+            n = n < N ? n : N - 1;
+            rw[i] = kk < K ? *reinterpret_cast<const uint4*>(we + (size_t)n * K + kk) : make_uint4(0, 0, 0, 0);
+        }
+    };
+    auto sstore = [&](int stage, const uint4* ra, const uint4* rw) {
+        uint16_t* sa = smem + stage * STAGE;
+        uint16_t* sw = sa + BM * STRIDE;
+#pragma unroll
+        for (int i = 0; i < A_CH; i++) {
+            const int c = tid + i * NT;
+            *reinterpret_cast<uint4*>(sa + (c / CPR) * STRIDE + (c % CPR) * 8) = ra[i];
+        }
+#pragma unroll
+        for (int i = 0; i < W_CH; i++) {
+            const int c = tid + i * NT;
+            *reinterpret_cast<uint4*>(sw + (c / CPR) * STRIDE + (c % CPR) * 8) = rw[i];
+        }
+    };
+    auto compute = [&](int stage) {
+        const uint16_t* sa = smem + stage * STAGE + (wm * TM + (lane & 31)) * STRIDE + (lane >> 5) * 8;
+        const uint16_t* sw = smem + stage * STAGE + (BM + wn * TN + (lane & 31)) * STRIDE + (lane >> 5) * 8;
+#pragma unroll
+        for (int kk = 0; kk < BK; kk += 16) {
+            MFrag fa[FM], fw[FN];
+#pragma unroll
+            for (int j = 0; j < FN; j++) fw[j].u = *reinterpret_cast<const uint4*>(sw + j * 32 * STRIDE + kk);
+#pragma unroll
+            for (int i = 0; i < FM; i++) {
+                // an expert's last tile is seldom full: a wave multiplies only the runs of 32 rows that hold any
+                if (wm * TM + 32 * i >= nr) continue;
+                fa[i].u = *reinterpret_cast<const uint4*>(sa + i * 32 * STRIDE + kk);
+#pragma unroll
+                for (int j = 0; j < FN; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[i].v, fw[j].v, acc[i][j], 0, 0, 0);
+            }
+        }
+    };
+    const int nk = (K + BK - 1) / BK;
+#pragma unroll
+    for (int p = 0; p < PF; p++)
+        if (p < nk) gload(ra[p], rw[p], p * BK);
+    sstore(0, ra[0], rw[0]);
+    if (PF < nk) gload(ra[0], rw[0], PF * BK);
+    __syncthreads();
+    for (int t0 = 0; t0 < nk; t0 += PF) {
+#pragma unroll
+        for (int p = 0; p < PF; p++) {                       // tile t0 + p: the register sets are constants here
+            const int t = t0 + p;
+            if (t >= nk) break;
+            compute(t & 1);
+            if (t + 1 < nk) {
+                sstore((t + 1) & 1, ra[(p + 1) % PF], rw[(p + 1) % PF]);
+                if (t + 1 + PF < nk) gload(ra[(p + 1) % PF], rw[(p + 1) % PF], (t + 1 + PF) * BK);
+            }
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < FM; i++) {
+#pragma unroll
+        for (int r = 0; r < 16; r++) {
+            const int row = wm * TM + 32 * i + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
+            if (row >= nr) continue;
+            const int pair = pair_s[row];
+            const float sc = pair_scale ? pair_scale[pair] : 1.f;
+            const size_t orow = out_by_pair ? (size_t)pair : (size_t)(r0 + row);
+#pragma unroll
+            for (int j = 0; j < FN; j++) {
+                const int n = n0 + wn * TN + 32 * j + (lane & 31);
+                if (n < N) out[orow * ldo + n] = from_f32<TO>(hfa_act_apply(act, acc[i][j][r]) * sc);
             }
         }
     }
 }
 
 extern "C" int hfa_moe_tile_rows(int dtype, int w_dtype, int n_pairs, int n_experts, int N, int K) {
-    if (dtype == HFA_BF16 && w_dtype == HFA_BF16 && K % 16 == 0 && N % 32 == 0) return n_pairs >= 48 * n_experts ? 64 : 32;
+    if (dtype == HFA_BF16 && w_dtype == HFA_BF16 && K % 16 == 0 && N % 32 == 0)
+        return n_pairs >= 96 * n_experts ? 128 : n_pairs >= 48 * n_experts ? 64 : 32;
     return PM;
 }
 
@@ -316,8 +490,36 @@ extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const 
                     (w_dtype == HFA_F32 || w_dtype == HFA_BF16), "moe_gemm: unknown dtype");
     HFA_REQUIRE(act >= 0 && act <= HFA_ACT_RELU2 && a_div >= 0, "moe_gemm: bad activation or divisor");
     const bool mfma = !force_plain && dtype == HFA_BF16 && w_dtype == HFA_BF16 && K % 16 == 0 && N % 32 == 0 && lda % 8 == 0 &&
-                      (tile_rows == 32 || tile_rows == 64) && ((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0;
-    if (mfma) {
+                      (tile_rows == 32 || tile_rows == 64 || tile_rows == 128) && ((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0;
+    if (mfma && tile_rows >= 64) {
+        dim3 grid(max_tiles, (N + 127) / 128);
+#define MOE_LDS(BM, BN, BK, TO)                                                                                           \
+    do {                                                                                                                  \
+        auto kernel = moe_gemm_lds_kernel<BM, BN, BK, TO>;                                                                \
+        constexpr int SMEM = 2 * (BM + BN) * (BK + 8) * 2;                                                                \
+        static bool configured = false;                                                                                   \
+        if (!configured) {                                                                                                \
+            if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM) != hipSuccess) {  \
+                hfa_set_error("moe_gemm: cannot reserve %d bytes of LDS", SMEM);                                          \
+                return 2;                                                                                                 \
+            }                                                                                                             \
+            configured = true;                                                                                            \
+        }                                                                                                                 \
+        kernel<<<grid, 256, SMEM, stream>>>((const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles, n_tiles, (TO*)out, ldo, \
+                                            out_by_pair, pair_scale, act, N, K);                                          \
+    } while (0)
+        if (tile_rows == 128) { if (out_dtype == HFA_F32) MOE_LDS(128, 128, 32, float); else MOE_LDS(128, 128, 32, bf16); }
+        else { if (out_dtype == HFA_F32) MOE_LDS(64, 128, 32, float); else MOE_LDS(64, 128, 32, bf16); }
+#undef MOE_LDS
+    } else if (mfma && K % 64 == 0) {
+        dim3 grid(max_tiles, (N + 31) / 32);
+        if (out_dtype == HFA_F32)
+            moe_gemm_split_kernel<float><<<grid, 256, 0, stream>>>((const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles,
+                                                                   n_tiles, (float*)out, ldo, out_by_pair, pair_scale, act, N, K);
+        else
+            moe_gemm_split_kernel<bf16><<<grid, 256, 0, stream>>>((const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles,
+                                                                  n_tiles, (bf16*)out, ldo, out_by_pair, pair_scale, act, N, K);
+    } else if (mfma) {
         const int cn = N % 256 == 0 && N >= 512 ? 2 : 1;
         dim3 grid(max_tiles, (N + 128 * cn - 1) / (128 * cn));
 #define MOE_ARGS (const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles, n_tiles
@@ -327,8 +529,7 @@ extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const 
         if (out_dtype == HFA_F32) moe_gemm_mfma_kernel<RM, CN, float><<<grid, 256, 0, stream>>>(MOE_ARGS, (float*)out, MOE_TAIL); \
         else moe_gemm_mfma_kernel<RM, CN, bf16><<<grid, 256, 0, stream>>>(MOE_ARGS, (bf16*)out, MOE_TAIL);                  \
     } while (0)
-        if (tile_rows == 64) { if (cn == 2) MOE_GO(2, 2); else MOE_GO(2, 1); }
-        else { if (cn == 2) MOE_GO(1, 2); else MOE_GO(1, 1); }
+        if (cn == 2) MOE_GO(1, 2); else MOE_GO(1, 1);
 #undef MOE_GO
 #undef MOE_ARGS
 #undef MOE_TAIL
@@ -361,12 +562,28 @@ __global__ void moe_combine_kernel(const float* __restrict__ y, float* __restric
         x[i] += s;
     }
 }
+// the same, four columns a thread (width a multiple of 4)
+__global__ void moe_combine4_kernel(const float4* __restrict__ y, float4* __restrict__ x, int top, int width4, size_t total4) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total4; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t t = i / width4, c = i % width4;
+        float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int k = 0; k < top; k++) {
+            const float4 v = y[(t * top + k) * width4 + c];
+            s.x += v.x; s.y += v.y; s.z += v.z; s.w += v.w;
+        }
+        float4 o = x[i];
+        o.x += s.x; o.y += s.y; o.z += s.z; o.w += s.w;
+        x[i] = o;
+    }
+}
 
 extern "C" int hfa_moe_combine(const float* y, float* x, int n_tokens, int top, int width, hipStream_t stream) {
     HFA_REQUIRE(y && x && n_tokens > 0 && top > 0 && width > 0, "moe_combine: bad arguments");
-    const size_t total = (size_t)n_tokens * width;
+    const bool vec = width % 4 == 0 && ((uintptr_t)y & 15) == 0 && ((uintptr_t)x & 15) == 0;
+    const size_t total = (size_t)n_tokens * width / (vec ? 4 : 1);
     const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
-    moe_combine_kernel<<<blocks, 256, 0, stream>>>(y, x, top, width, total);
+    if (vec) moe_combine4_kernel<<<blocks, 256, 0, stream>>>((const float4*)y, (float4*)x, top, width / 4, total);
+    else moe_combine_kernel<<<blocks, 256, 0, stream>>>(y, x, top, width, total);
     HFA_LAUNCH_CHECK("moe_combine");
     return 0;
 }

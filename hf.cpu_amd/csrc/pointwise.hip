@@ -11,6 +11,7 @@
 // the finished mean, so a row far from zero loses nothing), and a row's result does not depend on the rest of the
 // launch. As in hfa_rmsnorm, a product that left its result as partial sums (the residual sum of the layer before)
 // is finished first: x[r, :] += sum over splits + bias, written back.
+#define LN_KEEP 8          // values of the row that a thread keeps in registers between the passes
 template <typename TO>
 __global__ __launch_bounds__(1024) void layernorm_kernel(float* __restrict__ x, const float* __restrict__ w,
                                                         const float* __restrict__ b, TO* __restrict__ out,
@@ -18,11 +19,11 @@ __global__ __launch_bounds__(1024) void layernorm_kernel(float* __restrict__ x, 
                                                         const float* __restrict__ partial, int splits,
                                                         const float* __restrict__ pbias, int n_rows) {
     __shared__ float red[17];
-    const int r = blockIdx.x;
+    const int r = blockIdx.x, bd = blockDim.x;
     const int xr = rows ? rows[r] : r;
     float* src = x + (size_t)xr * width;
-    float sum = 0.f;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+    // the row's value at column i, with a deferred product's partial sums added (and written back) first
+    auto value = [&](int i) {
         float v = src[i];
         if (splits > 0) {
             for (int s0 = 0; s0 < splits; s0 += LN_PLANE_BATCH) {
@@ -36,17 +37,37 @@ __global__ __launch_bounds__(1024) void layernorm_kernel(float* __restrict__ x, 
             if (pbias) v += pbias[i];
             src[i] = v;
         }
-        sum += v;
+        return v;
+    };
+    // Rows of up to LN_KEEP values a thread are read once; what lies beyond is read again in each pass.
+    float keep[LN_KEEP];
+    float sum = 0.f;
+#pragma unroll
+    for (int k = 0; k < LN_KEEP; k++) {
+        const int i = threadIdx.x + k * bd;
+        keep[k] = i < width ? value(i) : 0.f;
+        sum += keep[k];
     }
+    for (int i = threadIdx.x + LN_KEEP * bd; i < width; i += bd) sum += value(i);
     const float mean = block_sum(sum, red) / (float)width;      // the barriers inside also order the writes of x
     float sq = 0.f;
-    for (int i = threadIdx.x; i < width; i += blockDim.x) {
+#pragma unroll
+    for (int k = 0; k < LN_KEEP; k++) {
+        const float d = keep[k] - mean;
+        if ((int)threadIdx.x + k * bd < width) sq = fmaf(d, d, sq);
+    }
+    for (int i = threadIdx.x + LN_KEEP * bd; i < width; i += bd) {
         const float d = src[i] - mean;
         sq = fmaf(d, d, sq);
     }
     const float inv = 1.0f / sqrtf(block_sum(sq, red) / (float)width + eps);
     TO* dst = out + (size_t)r * width;
-    for (int i = threadIdx.x; i < width; i += blockDim.x)
+#pragma unroll
+    for (int k = 0; k < LN_KEEP; k++) {
+        const int i = threadIdx.x + k * bd;
+        if (i < width) dst[i] = from_f32<TO>(fmaf((keep[k] - mean) * inv, w[i], b ? b[i] : 0.f));
+    }
+    for (int i = threadIdx.x + LN_KEEP * bd; i < width; i += bd)
         dst[i] = from_f32<TO>(fmaf((src[i] - mean) * inv, w[i], b ? b[i] : 0.f));
 }
 
@@ -56,7 +77,7 @@ extern "C" int hfa_layernorm(float* x, const float* w, const float* b, void* out
     HFA_REQUIRE(x && w && out && n_rows > 0 && width > 0, "layernorm: bad arguments");
     HFA_REQUIRE(out_dtype == HFA_F32 || out_dtype == HFA_BF16, "layernorm: unknown dtype %d", out_dtype);
     HFA_REQUIRE(splits == 0 || (partial && !rows), "layernorm: partial sums go with all rows in order");
-    int threads = width >= 4096 ? 1024 : width >= 1024 ? 512 : width >= 256 ? 256 : 64;
+    const int threads = width >= 8192 ? 1024 : width >= 2048 ? 512 : width >= 512 ? 256 : width >= 128 ? 128 : 64;
     if (out_dtype == HFA_F32)
         layernorm_kernel<float><<<n_rows, threads, 0, stream>>>(x, w, b, (float*)out, rows, width, eps, partial, splits,
                                                                 partial_bias, x_rows);
@@ -68,19 +89,12 @@ extern "C" int hfa_layernorm(float* x, const float* w, const float* b, void* out
 }
 
 // ---- activations ------------------------------------------------------------------------
-__device__ __forceinline__ float act_apply(int kind, float z) {
-    if (kind == HFA_ACT_GELU_ERF) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
-    if (kind == HFA_ACT_GELU_TANH) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
-    if (kind == HFA_ACT_RELU2) { const float r = fmaxf(z, 0.f); return r * r; }
-    return z;
-}
-
 template <typename T>
 __global__ void activation_kernel(const T* __restrict__ in, int ldi, T* __restrict__ out, int ldo, int width, int kind,
                                   size_t total) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t r = i / width, c = i % width;
-        out[r * ldo + c] = from_f32<T>(act_apply(kind, to_f32(in[r * ldi + c])));
+        out[r * ldo + c] = from_f32<T>(hfa_act_apply(kind, to_f32(in[r * ldi + c])));
     }
 }
 

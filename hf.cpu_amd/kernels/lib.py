@@ -18,7 +18,7 @@ _SIGNATURES = {
     "hfa_rmsnorm": [P, P, P, I, P, I, I, F, P, I, P, P],
     "hfa_gemm": [P, I, I, P, I, I, P, P, I, I, I, I, I, I, I, P, c_size_t, I, P, I, P],
     "hfa_gemm_finish": [P, I, P, P, I, I, I, I, I, I, P],
-    "hfa_gemm_rows": [I, P, I, P, I, I, I, I, P, P, I, F, F, P, I, I, P, I, P, P, P, I, P, I, P],
+    "hfa_gemm_rows": [I, P, I, P, I, I, I, I, P, P, I, F, F, P, I, I, I, P, I, P, P, P, I, P, I, P],
     "hfa_gemm_rows_supports": [I, I, I, I, I, I],
     "hfa_rope_store": [P, I, I, P, P, I, I, I, I, I, P, P, P, I, I, P, I, P, P],
     "hfa_paged_attention": [P, I, I, P, P, I, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, I, F, P, P, c_size_t, I, P],

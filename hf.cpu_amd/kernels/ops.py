@@ -327,7 +327,7 @@ class Ops:
             return mode if out.dtype == torch.bfloat16 and bias is None else None
         return mode
 
-    def _rows_call(self, mode, a, w, N, bias, scaled=None, out=None, x=None, ssq_out=None, g=None, xg=None, act=None):
+    def _rows_call(self, mode, a, w, N, bias, scaled=None, out=None, x=None, ssq_out=None, g=None, xg=None, act=None, out_act=0):
         M, K = a.shape
         null = ctypes.c_void_p(None)
 
@@ -336,7 +336,7 @@ class Ops:
         self._check(self.lib.hfa_gemm_rows(
             mode, a.data_ptr(), _rows(a, "gemm a"), w.data_ptr(), _rows(w, "gemm w"), M, N, K, ptr(bias),
             ptr(None if scaled is None else scaled.ssq), self.rows_parts, 1.0 / K, 0.0 if scaled is None else scaled.eps,
-            ptr(out), 0 if out is None else _rows(out, "gemm out"), 0 if out is None else _code(out),
+            ptr(out), 0 if out is None else _rows(out, "gemm out"), 0 if out is None else _code(out), int(out_act),
             ptr(x), 0 if x is None else _rows(x, "gemm out"), ptr(ssq_out), ptr(g),
             ptr(xg), 0 if xg is None else _rows(xg, "norm out"), ptr(act), 0 if act is None else _rows(act, "gemm out"),
             self._stream()))
@@ -405,11 +405,13 @@ class Ops:
         partial sums for the next kernel that reads ``out`` (see the module's text).
         ``swiglu``: w's rows come in blocks of 32 gate, 32 up (``interleave_gate_up``) and
         out = silu(gate) * up has half as many columns. ``activation``: ``out = act(a @ w.T + bias)`` (see ``activation``)."""
+        act = 0
         if activation is not None:
-            if accumulate or swiglu:
-                fail(EINVAL, "gemm: an activation goes with a plain output")
-            self.gemm(a, w, out, bias=bias)
-            return self.activation(activation, out, out)
+            if accumulate or swiglu or defer:
+                fail(EINVAL, "gemm: an activation goes with a plain output that is finished at once")
+            if activation not in self.ACTIVATIONS:
+                fail(ENOTSUP, f"activation '{activation}' is not one of {', '.join(sorted(self.ACTIVATIONS))}")
+            act = self.ACTIVATIONS[activation]           # the product's last lines apply it
         self.settle()
         lda, ldw, ldo = _rows(a, "gemm a"), _rows(w, "gemm w"), _rows(out, "gemm out")
         M, K = a.shape
@@ -439,7 +441,7 @@ class Ops:
                 self._rows_call(0, a, w, N, bias, scaled=scaled, out=plane)
                 self._pending = Pending(out, 1, None, False)
             else:
-                self._rows_call(0, a, w, N, bias, scaled=scaled, out=out)
+                self._rows_call(0, a, w, N, bias, scaled=scaled, out=out, out_act=act)
             return
         if scaled is not None:
             self._whole(a)
@@ -449,7 +451,7 @@ class Ops:
         self._splits_out.value = 0
         self._check(self.lib.hfa_gemm(a.data_ptr(), _code(a), lda, w.data_ptr(), _code(w), ldw,
                                       None if bias is None else bias.data_ptr(), out.data_ptr(), _code(out), ldo,
-                                      1 if accumulate else 0, 1 if swiglu else 0, M, N, K, self.workspace.data_ptr(),
+                                      1 if accumulate else 0, 1 + act if act else 1 if swiglu else 0, M, N, K, self.workspace.data_ptr(),
                                       self.workspace.numel(), 1 if defer else 0, ctypes.byref(self._splits_out),
                                       1 if self.force_plain_gemm else 0, self._stream()))
         if self._splits_out.value:

@@ -58,6 +58,25 @@ def test_activations_and_soft_cap(ops32, dtype):
     assert np.max(np.abs(x.cpu().numpy() - want)) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("M,N,K", [(1, 256, 512), (8, 384, 256), (16, 4608, 3584), (20, 1000, 1024), (33, 200, 1000), (100, 256, 512),
+                                   (128, 1024, 2048), (300, 512, 256), (2048, 1024, 512), (700, 8192, 2048), (5, 100, 33)])
+def test_product_with_an_activation_in_its_last_lines(ops32, ops16, dtype, M, N, K):
+    """``gemm(..., activation=)`` at shapes that go to every product kernel (few rows that finish their outputs, K cut
+    over waves and blocks, tiles through LDS, the plain kernel), with a bias, against the plain product and function."""
+    ops = ops32 if dtype == torch.float32 else ops16
+    rng = np.random.default_rng(M + N + K)
+    a = rounded(rng.standard_normal((M, K)).astype(np.float32), dtype)
+    w = rounded((rng.standard_normal((N, K)) / math.sqrt(K) * 2).astype(np.float32), dtype)
+    bias = rng.standard_normal(N).astype(np.float32)
+    z = a @ w.T + bias
+    for kind, want in (("gelu_erf", pg.gelu_erf(z)), ("relu2", np.maximum(z, 0.0) ** 2)):
+        out = torch.empty((M, N), dtype=dtype, device="cuda")
+        ops.gemm(dev(a, dtype), dev(w, dtype), out, bias=dev(bias), activation=kind)
+        err = np.max(np.abs(out.float().cpu().numpy() - want) / (1 + np.abs(want)))
+        assert err <= (2e-5 if dtype == torch.float32 else 0.01), f"{kind}: {err:.3e}"
+
+
 @pytest.mark.parametrize("E,top,groups,keep", [(8, 3, 2, 1), (6, 2, 3, 2), (5, 1, 1, 1), (4, 4, 4, 4), (16, 3, 4, 2),
                                                (64, 6, 8, 3), (128, 8, 1, 1), (7, 7, 1, 1), (12, 1, 12, 1), (256, 8, 8, 4)])
 def test_router(ops32, E, top, groups, keep):
@@ -87,7 +106,8 @@ def test_router_drops_the_experts_of_groups_that_lose(ops32):
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,W,F,E,top", [(1, 48, 40, 6, 2), (7, 256, 128, 8, 1), (300, 256, 64, 4, 4), (33, 128, 32, 16, 3),
-                                         (700, 256, 128, 8, 2), (5, 100, 24, 5, 1), (64, 512, 256, 32, 4)])
+                                         (700, 256, 128, 8, 2), (5, 100, 24, 5, 1), (64, 512, 256, 32, 4), (100, 256, 128, 4, 2),
+                                         (900, 384, 96, 3, 1)])
 def test_experts(ops32, ops16, dtype, T, W, F, E, top):
     """The experts' weighted sum for given choices, through the plan and the grouped products, against a loop."""
     ops = ops32 if dtype == torch.float32 else ops16
