@@ -113,8 +113,11 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     int k_begin = first_visible(pos_first, window, mask_chunk);
     int k_end = hi;
     if (SPLIT) {
-        k_begin = k_begin > chunk * chunk_keys ? k_begin : chunk * chunk_keys;
-        k_end = k_end < (chunk + 1) * chunk_keys - 1 ? k_end : (chunk + 1) * chunk_keys - 1;
+        // Under a mask by chunks the tile's keys begin far into the sequence: the cuts are then counted from the first
+        // key block that the tile sees, not from key 0 (whose chunks would mostly hold nothing).
+        const int c_lo = (mask_chunk > 0 ? k_begin / KB * KB : 0) + chunk * chunk_keys;
+        k_begin = k_begin > c_lo ? k_begin : c_lo;
+        k_end = k_end < c_lo + chunk_keys - 1 ? k_end : c_lo + chunk_keys - 1;
     }
     // visible keys of this lane's column: [vlo, vhi]
     int vlo = first_visible(pos, window, mask_chunk) > k_begin ? first_visible(pos, window, mask_chunk) : k_begin;
@@ -535,7 +538,8 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     // of the key block) and leaves maximum, sum and unscaled output for attn_merge_kernel; a chunk
     // that holds none of the tile's keys leaves an empty record.
     if (n_chunks > 1) {
-        const int c_lo = blockIdx.z * chunk_keys, c_hi = c_lo + chunk_keys - 1;
+        // (under a mask by chunks, counted from the first key block that the tile sees: see attn_mfma_kernel)
+        const int c_lo = (mask_chunk > 0 ? k_begin / KB * KB : 0) + blockIdx.z * chunk_keys, c_hi = c_lo + chunk_keys - 1;
         k_begin = k_begin > c_lo ? k_begin : c_lo;
         hi = hi < c_hi ? hi : c_hi;
     }
@@ -923,15 +927,19 @@ static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
     // chunks' results together (portions of a few hundred tokens far into a long prompt).
     int n_chunks = 1, chunk_keys = a.max_seq_len;
     const long blocks = (long)a.n_kv_heads * ((a.n_tokens + tile_tokens - 1) / tile_tokens);
-    if (blocks < 2 * cus && a.max_seq_len >= 512 && a.workspace != nullptr) {
+    // the keys that one tile can see: all of the sequence, or a masking chunk and the tile's own tokens (and the key
+    // block that the cuts are aligned to); the cuts are made over these
+    int reach = a.max_seq_len;
+    if (a.mask_chunk > 0 && a.mask_chunk + tile_tokens + KB < reach) reach = a.mask_chunk + tile_tokens + KB;
+    if (blocks < 2 * cus && reach >= 512 && a.workspace != nullptr) {
         long want = (2 * cus + blocks - 1) / blocks;
-        if (want > a.max_seq_len / 256) want = a.max_seq_len / 256;
+        if (want > reach / 256) want = reach / 256;
         if (want > MERGE_MAX_CHUNKS) want = MERGE_MAX_CHUNKS;
         const size_t per_chunk = (size_t)a.n_tokens * a.n_heads * (a.head_dim + 2) * sizeof(float);
         if ((size_t)want * per_chunk > a.workspace_bytes) want = (long)(a.workspace_bytes / per_chunk);
         if (want > 1) {
-            chunk_keys = (int)((a.max_seq_len + want - 1) / want + 63) / 64 * 64;
-            n_chunks = (a.max_seq_len + chunk_keys - 1) / chunk_keys;
+            chunk_keys = (int)((reach + want - 1) / want + 63) / 64 * 64;
+            n_chunks = (reach + chunk_keys - 1) / chunk_keys;
         }
     }
     if (n_chunks > 1) {
@@ -999,9 +1007,11 @@ int attn_mfma_launch(const AttnArgs& a) {
         int want = (int)((fill + waves - 1) / waves);
         const int most = (span + 127) / 128;
         if (want > most) want = most;
-        chunk_keys = ((a.max_seq_len + want - 1) / want + KB - 1) / KB * KB;
+        // under a mask by chunks the cuts are counted from the tile's first key block: they cover what a tile can see
+        const int reach = a.mask_chunk > 0 && span + KB < a.max_seq_len ? span + KB : a.max_seq_len;
+        chunk_keys = ((reach + want - 1) / want + KB - 1) / KB * KB;
         if (chunk_keys < 64) chunk_keys = 64;
-        n_chunks = (a.max_seq_len + chunk_keys - 1) / chunk_keys;
+        n_chunks = (reach + chunk_keys - 1) / chunk_keys;
         const size_t need = (size_t)a.n_tokens * a.n_heads * n_chunks * (a.head_dim + 2) * sizeof(float);
         if (n_chunks < 2 || n_chunks > MERGE_MAX_CHUNKS || need > a.workspace_bytes) {
             n_chunks = 1;
