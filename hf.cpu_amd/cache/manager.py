@@ -6,14 +6,16 @@ lazily by ``kv_reserve``, src/model.c:309-330, and freed only with the context,
 src/model.c:217-230). Here pages come from shared pools:
 
 * Schedule entries whose mixers ask for paged storage are put into **groups** by what
-  they ask for (row widths and window). A group has its own page ids, its own pool and,
+  they ask for (row widths, window, masking chunk and what their readers see). A group has its own page ids, its own pool and,
   per request, its own block table; all entries of a group use the same page id for the
   same tokens, each in its own memory.
 * A request's block ``b`` of a group covers positions ``b * page_tokens ..``; the table
   is indexed by absolute block number.
 * Pages go back to the pool when the request is released, and, in a group with a
   window ``W``, as soon as every position on the page is ``<= next_pos - W`` for the
-  request's next position: no later query can see them.
+  request's next position: no later query can see them. A group whose mixers mask by chunks gives
+  back the pages that lie wholly before the current chunk's start; where other mixers read the same
+  storage (``PagedKV.readers``), a page goes back only when none of them can see it any more.
 * ``fork`` gives a new request the cache of another (src/model.c:271-301): whole pages are
   shared and counted, the last, partly filled page is copied, because both will write there.
   A shared page is never written: a request writes only at and beyond its own length.
@@ -36,6 +38,7 @@ class Group:
     k_width: int
     v_width: int
     window: int
+    need: object = None                             # the PagedKV that says which rows may be forgotten
     entries: list = field(default_factory=list)     # schedule entries that store here
 
 
@@ -65,10 +68,10 @@ class CacheManager:
         by_key = {}
         for i, need in enumerate(needs):
             if isinstance(need, PagedKV):
-                key = (need.k_width, need.v_width, need.window)
+                key = (need.k_width, need.v_width, need.window, need.mask_chunk, tuple(sorted(set(need.readers))))
                 if key not in by_key:
                     by_key[key] = len(self.groups)
-                    self.groups.append(Group(len(self.groups), *key))
+                    self.groups.append(Group(len(self.groups), need.k_width, need.v_width, need.window, need))
                 self.groups[by_key[key]].entries.append(i)
                 self.entry_group.append(by_key[key])
             else:
@@ -141,9 +144,7 @@ class CacheManager:
     # ---- pages ---------------------------------------------------------------
     def _first_needed_block(self, group, next_pos):
         """Blocks before this one hold only keys that no query at ``next_pos`` or later sees."""
-        if group.window <= 0:
-            return 0
-        return max(0, next_pos - group.window + 1) // self.page_tokens
+        return group.need.first_kept(next_pos) // self.page_tokens
 
     def pages_needed(self, req_id, n_new):
         """Per group, the pages ``reserve(req_id, n_new)`` would take (the request may be
@@ -206,7 +207,7 @@ class CacheManager:
         h.length += n_new
         h.reserved = 0
         for g in self.groups:
-            if g.window > 0:
+            if g.need.first_kept(h.length) > 0:
                 table = h.tables[g.index]
                 stop = min(self._first_needed_block(g, h.length), len(table))
                 gone = [table[b] for b in range(stop) if table[b] >= 0]

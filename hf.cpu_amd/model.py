@@ -131,6 +131,11 @@ class Model:
                     raise TypeError(f"{type(part).__name__}.cache_need() returned {need!r}")
                 slots[name] = len(needs)
                 needs.append(need)
+                if e.cache_of is not None and hasattr(part, "reads_cache"):
+                    # what the reader sees of the other entry's storage decides with it how long rows are kept
+                    k = self.cache_slots[e.cache_of].get(name)
+                    if k is not None and isinstance(needs[k], PagedKV):
+                        needs[k] = part.reads_cache(needs[k])
             self.cache_slots.append(slots)
         return needs
 

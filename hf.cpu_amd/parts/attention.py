@@ -82,7 +82,11 @@ class Attention(Part):
         if not self.own_kv:
             fail(EINVAL, f"attention '{self.prefix}' has no keys and values of its own: its schedule entry must read "
                          "another entry's cache")
-        return PagedKV(self.KD, self.VD, self.window)
+        return PagedKV(self.KD, self.VD, self.window, self.mask_chunk)
+
+    def reads_cache(self, need):
+        """``need`` of the mixer whose storage this one reads, widened by what this one sees of it."""
+        return PagedKV(need.k_width, need.v_width, need.window, need.mask_chunk, need.readers + ((self.window, self.mask_chunk),))
 
     def bind(self, params, ops):
         p, nm = self.prefix, self.names

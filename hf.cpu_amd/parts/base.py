@@ -36,10 +36,22 @@ class ParamSpec:
 class PagedKV:
     """A mixer's need for storage that grows with the sequence: one key row and one
     value row per token, kept for every earlier token (``window == 0``) or for the
-    last ``window`` tokens only."""
+    last ``window`` tokens only; with ``mask_chunk > 0`` only from the start of the current run of
+    ``mask_chunk`` positions (counted from 0). ``readers``: the (window, mask_chunk) of every other
+    mixer that reads this storage (schedule entries with ``cache_of``): a row is kept while any of
+    them, or the owner, can still see it."""
     k_width: int
     v_width: int
     window: int = 0
+    mask_chunk: int = 0
+    readers: tuple = ()
+
+    def first_kept(self, next_pos):
+        """The first position that a query at ``next_pos`` or later can see, for the owner or any reader."""
+        def first(window, chunk):
+            lo = max(0, next_pos - window + 1) if window > 0 else 0
+            return max(lo, next_pos - next_pos % chunk) if chunk > 0 else lo
+        return min(first(w, c) for w, c in ((self.window, self.mask_chunk),) + tuple(self.readers))
 
 
 @dataclass(frozen=True)

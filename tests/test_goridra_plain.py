@@ -95,3 +95,26 @@ def test_configuration_and_plan():
     bad = {**gh.SMALL, "layers": [dict(gh.SMALL["layers"][0], type="recurrent")]}
     with pytest.raises(EngineError):
         config_from_dict(bad)
+
+
+def test_pages_before_the_current_chunk_go_back_unless_a_reader_still_sees_them():
+    from hf_cpu_amd.cache import CacheManager
+    from hf_cpu_amd.parts.base import PagedKV
+    need = PagedKV(8, 8, 0, 24, readers=((0, 16),))
+    assert [need.first_kept(p) for p in (0, 15, 16, 23, 24, 31, 32, 47, 48, 50)] == [0, 0, 0, 0, 16, 16, 24, 24, 48, 48]
+    assert PagedKV(8, 8, 0, 24, readers=((0, 0),)).first_kept(1000) == 0          # a reader that sees everything keeps everything
+    assert PagedKV(8, 8, 30, 0, readers=((0, 16),)).first_kept(100) == 71         # a window and a reader's chunk: the earlier of the two
+    m = CacheManager([need, None], page_tokens=8, n_pages=7, n_slots=1, max_context=400)
+    m.admit("a")
+    at = 0
+    for n in [10, 3, 9, 1, 1, 7, 10, 2] * 7:
+        m.reserve("a", n)
+        m.commit("a", n)
+        at += n
+        table = m.held["a"].tables[0]
+        first = need.first_kept(at) // 8
+        assert all(p < 0 for p in table[:first]) and all(p >= 0 for p in table[first:])
+        m.check()
+    assert at > 7 * 8 * 5 and m.pools[0].reused > 0
+    m.release("a")
+    assert m.pools[0].n_held == 0
