@@ -406,6 +406,37 @@ def test_a_long_request_in_a_pool_that_holds_a_chunk_of_it(gpu, tiny, dtype):
     assert all(p.reused > 0 and p.n_held == 0 for p in engine.manager.pools)
 
 
+def test_trace_replay_program(gpu, tiny, tmp_path):
+    """bin/trace_run as a user calls it (pages of 16, four slots, a pool for the live requests only): a mixed trace in
+    fp32 against the plain implementation; in bf16 the same trace, where all rows but a router's near ties agree with it."""
+    import json
+    import os
+    import subprocess
+    import sys
+    name, cfg, d, reqs, want = tiny
+    steps = helpers.trace_mixed(reqs, seed=21)
+    places = helpers.wanted_places(steps)
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for dtype in ("float32", "bfloat16"):
+        out = tmp_path / dtype
+        r = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", d, "--dtype", dtype, "--out", str(out),
+                            "--max-tokens", str(helpers.max_live_tokens(steps))],
+                           input="".join(json.dumps(st) + "\n" for st in steps), text=True, capture_output=True, timeout=300)
+        assert r.returncode == 0, r.stderr
+        assert [w for w in r.stdout.split() if w != "done"] == [str(st["step"]) for st in steps]
+        got = {}
+        for st in steps:
+            if st["step"] in places:
+                rows = np.fromfile(out / f"{st['step']}.f32", dtype="<f4").reshape(len(places[st["step"]]), -1)
+                got.update(zip(places[st["step"]], rows))
+        assert len(got) == sum(len(t) for t in reqs.values())
+        if dtype == "float32":
+            helpers.compare(got, want, TOL[dtype], "trace_run " + dtype)
+        else:
+            far = sum(float(np.max(np.abs(row - want[r][pos]))) > TOL[dtype] * float(np.max(np.abs(want[r]))) for (r, pos), row in got.items())
+            assert far <= len(got) // 10, f"{far} of {len(got)} rows are far from the plain logits"
+
+
 def test_greedy_generation_through_the_session(gpu, tiny):
     """Greedy continuation of three prompts through Session.generate (the scheduler, the sampler, graphs): every token
     is the plain implementation's best, or within rounding of it."""
