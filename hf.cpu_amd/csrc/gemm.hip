@@ -23,7 +23,12 @@ extern "C" int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int 
     }
     if (pending_splits) *pending_splits = 0;
     GemmArgs g = {a, a_dtype, lda, w, w_dtype, ldw, bias, out, out_dtype, ldo, accumulate, epilogue, M, N, K, stream, act};
-    if (!force_plain && gemm_mfma_supports(g)) return gemm_mfma_launch(g, workspace, workspace_bytes, defer, pending_splits);
+    if (!force_plain && gemm_mfma_supports(g)) {
+        if (!act || out_dtype == HFA_BF16) return gemm_mfma_launch(g, workspace, workspace_bytes, defer, pending_splits);
+        g.act = 0;                            // a 32-bit output: the product, then the elementwise kernel
+        const int rc = gemm_mfma_launch(g, workspace, workspace_bytes, 0, pending_splits);
+        return rc ? rc : hfa_activation(out, ldo, out, ldo, out_dtype, M, N, act, stream);
+    }
     HFA_REQUIRE(epilogue == 0, "gemm: the gate/up epilogue exists only on the matrix-core path");
     const int rc = gemm_generic_launch(g);
     if (rc || !act) return rc;

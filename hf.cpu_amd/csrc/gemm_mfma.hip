@@ -42,6 +42,8 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 #define OUT_ACC 2
 #define OUT_PARTIAL 3
 #define OUT_SWIGLU 4      // columns come in blocks of 32 gate, 32 up; out[m, f] = silu(gate) * up as bf16
+#define OUT_BF16_ACT 5    // bf16(act(sum + bias)): a mode of its own, so that the kernels of the other modes hold no line of it
+#define IS_BF16_OUT(MODE) ((MODE) == OUT_BF16 || (MODE) == OUT_BF16_ACT)
 
 template <int BM, int BN, int BK, int WM, int WN>
 struct MfmaCfg {
@@ -96,8 +98,8 @@ __device__ __forceinline__ void gemm_epilogue(floatx16 (&acc)[C::FM][C::FN], con
                 const int row = m0 + wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
                 if (row >= M) continue;
                 float v = acc[i][j][r] + b;
-                if ((MODE == OUT_BF16 || MODE == OUT_F32) && act) v = hfa_act_apply(act, v);
-                if (MODE == OUT_BF16) {
+                if (MODE == OUT_BF16_ACT) v = hfa_act_apply(act, v);
+                if (IS_BF16_OUT(MODE)) {
                     reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + col] = bf16_bits(v);
                 } else if (MODE == OUT_F32) {
                     reinterpret_cast<float*>(out)[(size_t)row * ldo + col] = v;
@@ -117,7 +119,7 @@ template <int BN, int MODE>
 struct DmaOut {
     static constexpr int PAIR = MODE == OUT_SWIGLU ? 2 : 1;      // 32 gate and 32 up columns give 32 results
     static constexpr int WIDTH = BN / PAIR, STRIDE = WIDTH + 8;
-    static constexpr int bytes(int bm) { return (MODE == OUT_BF16 || MODE == OUT_SWIGLU) ? bm * STRIDE * 2 : 0; }
+    static constexpr int bytes(int bm) { return (IS_BF16_OUT(MODE) || MODE == OUT_SWIGLU) ? bm * STRIDE * 2 : 0; }
 };
 
 // 16-bit results leave through LDS: a lane holds single columns, and a store of 2 bytes per lane
@@ -137,13 +139,13 @@ __device__ __forceinline__ void gemm_epilogue_rows(floatx16 (&acc)[C::FM][C::FN]
         for (int j = 0; j < C::FN; j += O::PAIR) {
             const int col = (wn * C::TN + j * 32) / O::PAIR + (lane & 31);      // within the block's tile
             const int gcol = n0 + wn * C::TN + j * 32 + (lane & 31);            // column of N (the gate's, if paired)
-            const float b = (MODE == OUT_BF16 && bias && gcol < N) ? bias[gcol] : 0.f;
+            const float b = (IS_BF16_OUT(MODE) && bias && gcol < N) ? bias[gcol] : 0.f;
 #pragma unroll
             for (int r = 0; r < 16; r++) {
                 const int row = wm * C::TM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r % 4);
                 float v = acc[i][j][r] + b;
                 if constexpr (MODE == OUT_SWIGLU) v = (v / (1.0f + expf(-v))) * acc[i][j + 1][r];
-                else if (act) v = hfa_act_apply(act, v);
+                else if constexpr (MODE == OUT_BF16_ACT) v = hfa_act_apply(act, v);
                 smem[row * O::STRIDE + col] = bf16_bits(v);
             }
         }
@@ -275,7 +277,7 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_mfma_kernel(
         }
     }
 
-    if constexpr (MODE == OUT_BF16 || MODE == OUT_SWIGLU) {
+    if constexpr (IS_BF16_OUT(MODE) || MODE == OUT_SWIGLU) {
         static_assert(DmaOut<BN, MODE>::bytes(BM) <= C::SMEM, "the tile of results fits the operand stages");
         if (rows_out) {                                      // uniform: the output allows 16-byte stores
             gemm_epilogue_rows<C, BM, BN, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane, tid, smem, act);
@@ -460,7 +462,7 @@ __global__ __launch_bounds__(WM* WN* WAVE) void gemm_dma_kernel(
     int t = 0;
     for (; t + AHEAD < nk; t++) step(t, std::true_type());
     for (; t < nk; t++) step(t, std::false_type());
-    if constexpr (MODE == OUT_BF16 || MODE == OUT_SWIGLU) {
+    if constexpr (IS_BF16_OUT(MODE) || MODE == OUT_SWIGLU) {
         gemm_epilogue_rows<C, BM, BN, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane, tid, smem, act);
     } else {
         gemm_epilogue<C, MODE>(acc, bias, out, ldo, M, N, m0, n0, wm, wn, lane, act);
@@ -477,14 +479,14 @@ __global__ void gemm_finish_kernel(const float* __restrict__ partial, int splits
     float v = 0.f;
     for (int s = 0; s < splits; s++) v += partial[(size_t)s * M * N + idx];
     if (bias) v += bias[col];
-    if ((MODE == OUT_BF16 || MODE == OUT_F32) && act) v = hfa_act_apply(act, v);
+    if (MODE == OUT_BF16_ACT) v = hfa_act_apply(act, v);
     if (MODE == OUT_SWIGLU) {                 // this thread holds a gate column; its up column is 32 further
         if ((col & 32) != 0) return;
         float up = 0.f;
         for (int s = 0; s < splits; s++) up += partial[(size_t)s * M * N + idx + 32];
         reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + (col / 64) * 32 + (col & 31)] =
             bf16_bits((v / (1.0f + expf(-v))) * up);
-    } else if (MODE == OUT_BF16)
+    } else if (IS_BF16_OUT(MODE))
         reinterpret_cast<uint16_t*>(out)[(size_t)row * ldo + col] = bf16_bits(v);
     else if (MODE == OUT_F32)
         reinterpret_cast<float*>(out)[(size_t)row * ldo + col] = v;
@@ -539,7 +541,7 @@ static int launch_cfg(const GemmArgs& g, void* out, int splits, int k_per_split)
     const int tiles_m = (g.M + BM - 1) / BM, tiles_n = (g.N + BN - 1) / BN;
     dim3 grid(tiles_m * tiles_n, 1, splits);
     const int n_out = MODE == OUT_SWIGLU ? g.N / 2 : g.N;
-    const int rows_out = (MODE == OUT_BF16 || MODE == OUT_SWIGLU) && g.ldo % 8 == 0 && n_out % 8 == 0 && ((uintptr_t)out & 15) == 0;
+    const int rows_out = (IS_BF16_OUT(MODE) || MODE == OUT_SWIGLU) && g.ldo % 8 == 0 && n_out % 8 == 0 && ((uintptr_t)out & 15) == 0;
     kernel<<<grid, C::NT, C::SMEM, g.stream>>>((const uint16_t*)g.a, g.lda, (const uint16_t*)g.w, g.ldw, g.bias, out,
                                               g.ldo, g.M, g.N, g.K, k_per_split, tiles_m, tiles_n, rows_out, g.act);
     HFA_LAUNCH_CHECK("gemm_mfma");
@@ -572,6 +574,7 @@ template <int BM, int BN, int BK, int WM, int WN, int STAGES>
 static int launch_dma(const GemmArgs& g, int mode, void* out, int splits, int k_per_split) {
     switch (mode) {
         case OUT_BF16: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_BF16>(g, out, splits, k_per_split);
+        case OUT_BF16_ACT: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_BF16_ACT>(g, out, splits, k_per_split);
         case OUT_F32: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_F32>(g, out, splits, k_per_split);
         case OUT_ACC: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_ACC>(g, out, splits, k_per_split);
         case OUT_PARTIAL: return launch_dma_cfg<BM, BN, BK, WM, WN, STAGES, OUT_PARTIAL>(g, out, splits, k_per_split);
@@ -586,6 +589,7 @@ template <int BM, int BN, int BK, int WM, int WN, int PF = (BM >= 128 ? 1 : 2)>
 static int launch_mode(const GemmArgs& g, int mode, void* out, int splits, int k_per_split) {
     switch (mode) {
         case OUT_BF16: return launch_cfg<BM, BN, BK, WM, WN, OUT_BF16, PF>(g, out, splits, k_per_split);
+        case OUT_BF16_ACT: return launch_cfg<BM, BN, BK, WM, WN, OUT_BF16_ACT, PF>(g, out, splits, k_per_split);
         case OUT_F32: return launch_cfg<BM, BN, BK, WM, WN, OUT_F32, PF>(g, out, splits, k_per_split);
         case OUT_ACC: return launch_cfg<BM, BN, BK, WM, WN, OUT_ACC, PF>(g, out, splits, k_per_split);
         case OUT_SWIGLU:
@@ -607,6 +611,8 @@ int gemm_finish_launch(const float* partial, int splits, const float* bias, void
     const int blocks = (int)((total + 255) / 256);
     if (mode == OUT_BF16)
         gemm_finish_kernel<OUT_BF16><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N, act);
+    else if (mode == OUT_BF16_ACT)
+        gemm_finish_kernel<OUT_BF16_ACT><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N, act);
     else if (mode == OUT_F32)
         gemm_finish_kernel<OUT_F32><<<blocks, 256, 0, stream>>>(partial, splits, bias, out, ldo, M, N, act);
     else if (mode == OUT_SWIGLU && !bias && N % 64 == 0 && ldo % 4 == 0 && ((uintptr_t)out & 7) == 0 && ((uintptr_t)partial & 15) == 0)
@@ -621,7 +627,7 @@ int gemm_finish_launch(const float* partial, int splits, const float* bias, void
 
 int gemm_mode_of(const GemmArgs& g) {
     if (g.epilogue == 1) return OUT_SWIGLU;
-    return g.accumulate ? OUT_ACC : (g.out_dtype == HFA_BF16 ? OUT_BF16 : OUT_F32);
+    return g.accumulate ? OUT_ACC : (g.out_dtype == HFA_BF16 ? (g.act ? OUT_BF16_ACT : OUT_BF16) : OUT_F32);
 }
 
 int gemm_mfma_launch(const GemmArgs& g, void* workspace, size_t workspace_bytes, int defer, int* pending_splits) {
