@@ -49,14 +49,14 @@ def test_rotation_turns_pairs_and_leaves_the_rest():
 
 
 def test_router_groups_and_weights():
-    z = np.array([[5.0, -9.0, -9.0, -9.0, 4.0, 4.1, 3.9, -9.0]])
+    z = np.array([[5.0, -9.0, -9.0, -9.0, -9.0, 4.0, 4.1, 3.9, -9.0, -9.0]])
     ids, w = pg.route(z, 3, 2, 1)
     assert ids.tolist() == [[0, 1, 2]] and abs(w.sum() - 1.0) < 1e-12
     ids, w = pg.route(z, 3, 2, 2)
-    assert ids.tolist() == [[0, 5, 4]]
+    assert ids.tolist() == [[0, 6, 5]]
     s = pg.softmax(z)[0]
-    assert np.allclose(w[0], s[[0, 5, 4]] / s[[0, 5, 4]].sum())
-    assert gh.choice_margin(s, 3, 2, 2) == pytest.approx(s[4] - s[6])
+    assert np.allclose(w[0], s[[0, 6, 5]] / s[[0, 6, 5]].sum())
+    assert gh.choice_margin(s, 3, 2, 2) == pytest.approx(s[5] - s[7])
 
 
 def test_a_layer_that_reads_another_layers_keys_and_values_and_a_layer_without_feed_forward(tmp_path):
