@@ -158,6 +158,10 @@ def chunk_attention(q, k, v, scale, size):
     (28, 4, 128, 16, 1024, [2100, 1025, 1024], [1, 1, 1]),                       # long chunks: the keys are cut over waves
     (4, 1, 64, 64, 80, [600], [600]),                                            # one prompt, whole; pages larger than a key block
     (2, 2, 128, 16, 200, [1100], [300]),                                         # a portion late in a prompt
+    (8, 2, 128, 16, 512, [1500], [1500]),                                        # few blocks, long chunks: a tile's keys cut over blocks
+    (8, 2, 64, 16, 700, [2000, 90], [400, 90]),                                  # the same for a portion that starts inside a chunk
+    (16, 2, 128, 32, 300, [1203, 2900, 301, 300, 599], [1, 1, 1, 1, 1]),         # decoded tokens at the first, second and last place of a chunk
+    (4, 4, 32, 8, 1000, [999, 1000, 1001, 2001], [40, 40, 40, 40]),              # portions across a chunk's border
 ])
 def test_attention_masked_by_chunks(ops32, ops16, dtype, H, G, D, page, size, lengths, q_lens):
     ops = ops32 if dtype == torch.float32 else ops16
@@ -454,6 +458,32 @@ def test_greedy_generation_through_the_session(gpu, tiny):
             row = pg.forward(pcfg, w, toks)[-1]
             assert row[int(np.argmax(row))] - row[t] <= 1e-4, f"token {i} = {t}, plain picks {int(np.argmax(row))}"
             toks.append(t)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_chunks_decoded_token_by_token(gpu, tmp_path, dtype):
+    """Chunks of several hundred positions: a decoded token's keys are cut over many waves, counted from its chunk's
+    start, in the kernel that also rotates and stores (the layer with keys of its own) and in the one that only attends
+    (its reader, with a shorter chunk); two requests decoded together across the border of both chunks."""
+    import hf_cpu_amd
+    cfg = dict(architecture="Goridra", vocab=300, width=128, logit_softcap=20.0, norm=dict(eps=1e-6), layers=[
+        gh.layer(gh.attention(4, 1, 64, 64, 64, 20000.0, 600), gh.dense(128)),
+        gh.layer(gh.attention(4, 1, 64, 64, 64, 20000.0, 350, kv_from=0), None)])
+    d = gh.make_model_dir(str(tmp_path / "m"), cfg, seed=4, stored="BF16")
+    reqs = gh.random_requests(cfg, [733, 1222], seed=2)
+    want = gh.plain_logits(d, reqs)
+    steps = []
+    heads = {r: len(t) - 45 for r, t in reqs.items()}
+    for r, t in reqs.items():
+        steps.append(helpers._step(len(steps), [(r, t[:heads[r]], [heads[r] - 1])]))
+    for i in range(45):
+        steps.append(helpers._step(len(steps), [(r, t[heads[r] + i:heads[r] + i + 1], [0]) for r, t in reqs.items()],
+                                   list(reqs) if i == 44 else []))
+    engine = hf_cpu_amd.load_engine(d, dtype=dtype, page_tokens=16, max_tokens=helpers.max_live_tokens(steps), max_seqs=2)
+    got = helpers.run_trace_in_engine(engine, steps)
+    assert len(got) == 2 * 46
+    helpers.compare(got, want, TOL[dtype], f"long chunks {dtype}")
+    engine.manager.check()
 
 
 def test_random_weights_and_a_second_configuration_of_the_same_files(gpu, tmp_path):
