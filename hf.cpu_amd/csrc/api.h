@@ -107,7 +107,8 @@ int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, 
 // the product left (`raw`, bias added): rotation of queries and keys (cos_sin: hfa_rope_table's output for the step's
 // tokens, [token][head_dim / 2 cosines, head_dim / 2 sines]; null: none), the store of the new key and value into
 // cache rows slot_map[t], and attention over the cache, in one kernel (plus the merge of key chunks): what
-// hfa_rope_store and hfa_paged_attention give one after the other. bf16 cache, matrix cores only: ask
+// hfa_rope_store and hfa_paged_attention give one after the other. With slot_map null the rows are [q] only and nothing
+// is stored (a layer that reads keys and values which another layer stored in this step). bf16 cache, matrix cores only: ask
 // hfa_decode_attention_supports first.
 int hfa_rope_table(const int* positions, const float* inv_freq, int half, float* out, int n_tokens, hipStream_t stream);
 int hfa_decode_attention_supports(int n_heads, int n_kv_heads, int head_dim, int rot_dim, int page_tokens, int kv_width,

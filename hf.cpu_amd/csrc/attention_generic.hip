@@ -164,7 +164,8 @@ extern "C" int hfa_decode_attention_supports(int n_heads, int n_kv_heads, int he
 // Attention of decoded tokens (one token a request) whose queries, new keys and new values are still the 32-bit rows
 // [q | k | v] that the product left (`raw`, row stride ld_raw, bias added): rotation of queries and keys, the store
 // of the new key and value into the cache rows slot_map[t], and attention over the cache in one kernel (and the merge
-// of the key chunks). cos_sin: hfa_rope_table's output for these tokens, or null for no rotation. Everything else as
+// of the key chunks). cos_sin: hfa_rope_table's output for these tokens, or null for no rotation. slot_map null: the
+// rows hold queries only ([q], a layer that reads the keys and values another layer has stored). Everything else as
 // in hfa_paged_attention, whose result with hfa_rope_store before it this equals.
 extern "C" int hfa_decode_attention(const float* raw, int ld_raw, const float* cos_sin, void* k_cache, void* v_cache,
                                     int kv_width, const int* slot_map, const int* block_table, int max_blocks,
@@ -172,10 +173,10 @@ extern "C" int hfa_decode_attention(const float* raw, int ld_raw, const float* c
                                     int max_seq_len, void* out, int ldo, int n_heads, int n_kv_heads, int head_dim,
                                     int page_tokens, int window, int mask_chunk, float scale, void* workspace,
                                     size_t workspace_bytes, hipStream_t stream) {
-    HFA_REQUIRE(raw && k_cache && v_cache && slot_map && block_table && token_slot && positions && q_start && out,
+    HFA_REQUIRE(raw && k_cache && v_cache && block_table && token_slot && positions && q_start && out,
                 "decode_attention: a null argument");
     HFA_REQUIRE(n_seqs > 0 && max_seq_len > 0 && max_blocks > 0 && window >= 0 && mask_chunk >= 0, "decode_attention: bad sizes");
-    HFA_REQUIRE(ld_raw >= (n_heads + 2 * n_kv_heads) * head_dim && ldo >= n_heads * head_dim && kv_width >= n_kv_heads * head_dim,
+    HFA_REQUIRE(ld_raw >= (n_heads + (slot_map ? 2 * n_kv_heads : 0)) * head_dim && ldo >= n_heads * head_dim && kv_width >= n_kv_heads * head_dim,
                 "decode_attention: a row stride is smaller than its row");
     AttnArgs a = {nullptr, 8, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot, positions, q_start,
                   n_seqs, 1, max_seq_len, out, ldo, n_seqs, n_heads, n_kv_heads, head_dim, page_tokens,

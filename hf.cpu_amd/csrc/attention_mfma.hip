@@ -146,7 +146,9 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
         const float* qsrc = row + my_head * D + half * 8;
         const float* ksrc = row + (H + g) * D + half * 8;
         const float* cp = cs ? cs + (size_t)my_tok * D + half * 8 : nullptr;
-        owns_new = k_begin <= hi && hi <= k_end;            // uniform: hi is the token's own position
+        // uniform: hi is the token's own position. Without slot_map the rows hold queries only (a layer that reads another
+        // layer's keys and values, which that layer has stored already): nothing is new.
+        owns_new = slot_map != nullptr && k_begin <= hi && hi <= k_end;
         const int slot = owns_new ? slot_map[my_tok] : 0;
         float vraw[NDB];
         if (owns_new && half == 0) {

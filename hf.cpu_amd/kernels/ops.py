@@ -480,13 +480,16 @@ class Ops:
         v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
         row_width = (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_head_dim
         pend = self._pending
+        # rows of q, k and v of a layer that stores, or rows of q alone of a layer that reads what another layer stored
+        stores = slot_map is not None and n_kv_heads > 0
+        reads = slot_map is None and n_kv_heads == 0 and getattr(cache, "k", None) is not None and cache.k.shape[1] % head_dim == 0
         if lazy and self.fuse_rows and pend is not None and pend.splits == 1 and pend.bias is None and not pend.accumulate \
                 and pend.out.data_ptr() == qkv.data_ptr() and pend.out.shape == qkv.shape and qkv.shape[1] == row_width \
-                and qkv.dtype == torch.bfloat16 and slot_map is not None and n_kv_heads and v_head_dim == head_dim \
+                and qkv.dtype == torch.bfloat16 and (stores or reads) and v_head_dim == head_dim \
                 and qkv.is_contiguous() and getattr(cache, "k", None) is not None and cache.k.dtype == torch.bfloat16 \
                 and cache.k.numel() < 1 << 32 and cache.k.shape[0] < 1 << 24 \
-                and self.lib.hfa_decode_attention_supports(n_heads, n_kv_heads, head_dim, rot_dim, cache.page_tokens,
-                                                           cache.k.shape[1], row_width, n_heads * head_dim):
+                and self.lib.hfa_decode_attention_supports(n_heads, n_kv_heads or cache.k.shape[1] // head_dim, head_dim, rot_dim,
+                                                           cache.page_tokens, cache.k.shape[1], row_width, n_heads * head_dim):
             self._lazy_rope = LazyRope((qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map,
                                         v_head_dim), qkv, cache)
             return
@@ -534,9 +537,10 @@ class Ops:
         lr = self._lazy_rope
         if lr is not None and lr.qkv.data_ptr() == q.data_ptr() and lr.cache is cache and slopes is None \
                 and step.max_q_len == 1 and step.n_seqs == q.shape[0] and not self.force_plain_attention \
-                and out.dtype == torch.bfloat16 and v_head_dim == head_dim and lr.args[4:7] == (n_heads, n_kv_heads, head_dim) \
+                and out.dtype == torch.bfloat16 and v_head_dim == head_dim and lr.args[4] == n_heads and lr.args[6] == head_dim \
+                and lr.args[5] in (0, n_kv_heads) and cache.k.shape[1] == n_kv_heads * head_dim \
                 and cache.k.numel() < 1 << 32 and cache.k.shape[0] < 1 << 24:
-            return self._decode_attention(lr, step, window, scale, out, mask_chunk)
+            return self._decode_attention(lr, step, window, scale, out, mask_chunk, n_kv_heads)
         self.settle()
         if slopes is not None and (slopes.dtype != torch.float32 or slopes.numel() != n_heads or not slopes.is_contiguous()
                                    or slopes.device != q.device):
@@ -583,10 +587,11 @@ class Ops:
         else:
             call(0, T, step.q_start, step.n_seqs, step.max_q_len)
 
-    def _decode_attention(self, lr, step, window, scale, out, mask_chunk=0):
+    def _decode_attention(self, lr, step, window, scale, out, mask_chunk=0, kv_heads=None):
         """Rotation, the store of the new keys and values and attention over the cache for decoded tokens, in one
         kernel: the queued ``rope_store`` (``lr``) and this call together."""
         qkv, positions, inv_freq, rot_dim, n_heads, n_kv_heads, head_dim, cache, slot_map, _ = lr.args
+        n_kv_heads = n_kv_heads or kv_heads          # a layer that only reads: its rows hold no keys, the cache says how many heads
         T = qkv.shape[0]
         table = None
         if rot_dim:
@@ -602,7 +607,7 @@ class Ops:
         self._pending = None                 # the 32-bit plane of q, k and v is read here
         self._check(self.lib.hfa_decode_attention(
             self.workspace.data_ptr(), qkv.shape[1], None if table is None else table.data_ptr(), cache.k.data_ptr(),
-            cache.v.data_ptr(), cache.k.shape[1], _ints(slot_map, "slot_map", T), g.block_table.data_ptr(),
+            cache.v.data_ptr(), cache.k.shape[1], None if slot_map is None else _ints(slot_map, "slot_map", T), g.block_table.data_ptr(),
             g.block_table.shape[1], _ints(step.token_slot, "token_slot", T), _ints(step.positions, "positions", T),
             _ints(step.q_start, "q_start", T + 1), T, step.max_seq_len, out.data_ptr(), _rows(out, "attention out"),
             n_heads, n_kv_heads, head_dim, cache.page_tokens, int(window), int(mask_chunk), float(scale),
