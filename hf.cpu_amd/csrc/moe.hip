@@ -348,26 +348,32 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
     }
 }
 
-// Matrix-core form for many rows an expert (prompt portions): a block of 2 x 2 waves owns BM rows of one expert x BN
+// Matrix-core form for many rows an expert (prompt portions): a block of WM x WN waves owns BM rows of one expert x BN
 // columns and walks K in steps of BK through two LDS stages, as gemm_mfma_kernel does for one matrix: the next tile
 // travels global -> registers while the current one is multiplied out of LDS, then registers -> LDS, one barrier a
 // step; LDS rows are padded by 8 elements so that the 16-byte fragment reads do not conflict. The rows of `a` are
 // gathered through row_pair (their source rows wait in LDS), so every operand element is read from memory once a
 // block instead of once a wave.
-template <int BM, int BN, int BK, typename TO>
-__global__ __launch_bounds__(256) void moe_gemm_lds_kernel(
+template <int BM, int BN, int BK, int WM, int WN, typename TO>
+__global__ __launch_bounds__(WM * WN * WAVE) void moe_gemm_lds_kernel(
     const uint16_t* __restrict__ a, int lda, int a_div, const uint16_t* __restrict__ w, const int* __restrict__ row_pair,
     const int* __restrict__ tiles, const int* __restrict__ n_tiles, TO* __restrict__ out, int ldo, int out_by_pair,
-    const float* __restrict__ pair_scale, int act, int N, int K) {
-    constexpr int STRIDE = BK + 8, NT = 256, CPR = BK / 8, A_CH = BM * CPR / NT, W_CH = BN * CPR / NT;
-    constexpr int TM = BM / 2, TN = BN / 2, FM = TM / 32, FN = TN / 32, STAGE = (BM + BN) * STRIDE;
+    const float* __restrict__ pair_scale, int act, int N, int K, int n_col_tiles) {
+    constexpr int STRIDE = BK + 8, NT = WM * WN * WAVE, CPR = BK / 8, A_CH = BM * CPR / NT, W_CH = BN * CPR / NT;
+    constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32, STAGE = (BM + BN) * STRIDE;
     static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0 && TM % 32 == 0 && TN % 32 == 0, "tiles spread evenly");
-    if ((int)blockIdx.x >= *n_tiles) return;
+    // Which (tile of rows, tile of columns): block ids are dealt round-robin to the 8 XCDs, each with an L2 of its own.
+    // The units, in the order (tile of rows, tile of columns), are cut into eight contiguous runs, one an XCD: the
+    // blocks that share a tile's rows, and the tiles that share an expert's matrix, then meet in one L2.
+    const int n_units = *n_tiles * n_col_tiles, per_xcd = (n_units + 7) / 8;
+    const int unit = (int)(blockIdx.x & 7) * per_xcd + (int)(blockIdx.x >> 3);
+    if ((int)(blockIdx.x >> 3) >= per_xcd || unit >= n_units) return;
+    const int tile = unit / n_col_tiles;
     extern __shared__ __attribute__((aligned(16))) uint16_t smem[];       // two stages of (BM + BN) x STRIDE elements
     __shared__ int src_s[BM], pair_s[BM];
-    const int e = tiles[3 * blockIdx.x], r0 = tiles[3 * blockIdx.x + 1], nr = tiles[3 * blockIdx.x + 2];
-    const int n0 = blockIdx.y * BN, tid = threadIdx.x, wave = tid / WAVE, lane = tid & (WAVE - 1);
-    const int wm = wave >> 1, wn = wave & 1;
+    const int e = tiles[3 * tile], r0 = tiles[3 * tile + 1], nr = tiles[3 * tile + 2];
+    const int n0 = (unit % n_col_tiles) * BN, tid = threadIdx.x, wave = tid / WAVE, lane = tid & (WAVE - 1);
+    const int wm = wave / WN, wn = wave % WN;
     for (int i = tid; i < BM; i += NT) {
         const int row = r0 + (i < nr ? i : 0);
         const int pair = row_pair[row];
@@ -492,10 +498,13 @@ extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const 
     const bool mfma = !force_plain && dtype == HFA_BF16 && w_dtype == HFA_BF16 && K % 16 == 0 && N % 32 == 0 && lda % 8 == 0 &&
                       (tile_rows == 32 || tile_rows == 64 || tile_rows == 128) && ((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0;
     if (mfma && tile_rows >= 64) {
-        dim3 grid(max_tiles, (N + 127) / 128);
-#define MOE_LDS(BM, BN, BK, TO)                                                                                           \
+        // (tiles of 128 x 256, on four waves and on eight, were measured and are slower at every size tried)
+        const int n_col_tiles = (N + 127) / 128;
+        HFA_REQUIRE((long)max_tiles * n_col_tiles + 8 < (1L << 31), "moe_gemm: too many tiles");
+        dim3 grid(((max_tiles * n_col_tiles + 7) / 8 + 1) * 8);      // every XCD's run of units has room, whatever the tile count
+#define MOE_LDS(BM, BN, BK, WM, WN, TO)                                                                                   \
     do {                                                                                                                  \
-        auto kernel = moe_gemm_lds_kernel<BM, BN, BK, TO>;                                                                \
+        auto kernel = moe_gemm_lds_kernel<BM, BN, BK, WM, WN, TO>;                                                        \
         constexpr int SMEM = 2 * (BM + BN) * (BK + 8) * 2;                                                                \
         static bool configured = false;                                                                                   \
         if (!configured) {                                                                                                \
@@ -505,11 +514,11 @@ extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const 
             }                                                                                                             \
             configured = true;                                                                                            \
         }                                                                                                                 \
-        kernel<<<grid, 256, SMEM, stream>>>((const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles, n_tiles, (TO*)out, ldo, \
-                                            out_by_pair, pair_scale, act, N, K);                                          \
+        kernel<<<grid, WM * WN * WAVE, SMEM, stream>>>((const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles, n_tiles,     \
+                                                       (TO*)out, ldo, out_by_pair, pair_scale, act, N, K, n_col_tiles);   \
     } while (0)
-        if (tile_rows == 128) { if (out_dtype == HFA_F32) MOE_LDS(128, 128, 32, float); else MOE_LDS(128, 128, 32, bf16); }
-        else { if (out_dtype == HFA_F32) MOE_LDS(64, 128, 32, float); else MOE_LDS(64, 128, 32, bf16); }
+        if (tile_rows == 128) { if (out_dtype == HFA_F32) MOE_LDS(128, 128, 32, 2, 2, float); else MOE_LDS(128, 128, 32, 2, 2, bf16); }
+        else { if (out_dtype == HFA_F32) MOE_LDS(64, 128, 32, 2, 2, float); else MOE_LDS(64, 128, 32, 2, 2, bf16); }
 #undef MOE_LDS
     } else if (mfma && K % 64 == 0) {
         dim3 grid(max_tiles, (N + 31) / 32);
