@@ -95,12 +95,13 @@ int hfa_attention_prompt_rows(void);
 // split over `workspace` when there are few queries; everything else, and everything when
 // `force_plain`, runs the plain kernel. `slopes` (one fp32 per query head, or null) is the hook for a position
 // encoding that enters the scores rather than the queries and keys: the score of key j for the query at p
-// becomes dot * scale + slopes[h] * (j - p); with slopes the plain kernel runs.
+// becomes dot * scale + slopes[h] * (j - p); with slopes the plain kernel runs. `sink` 1: the softmax has one more term
+// of score 0 that has no value, p_j = exp(s_j) / (1 + sum_i exp(s_i)) (every kernel takes it).
 int hfa_paged_attention(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache,
                         int kv_width, int v_width, const int* block_table, int max_blocks, const int* token_slot,
                         const int* positions, const int* q_start, int n_seqs, int max_q_len, int max_seq_len,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
-                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, void* workspace,
+                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, void* workspace,
                         size_t workspace_bytes, int force_plain, hipStream_t stream);
 
 // Decoded tokens (one a request) whose queries, new keys and new values are still the 32-bit rows [q | k | v] that
@@ -126,13 +127,48 @@ int hfa_layernorm(float* x, const float* w, const float* b, void* out, int out_d
                   int width, float eps, const float* partial, int splits, const float* partial_bias, int x_rows,
                   hipStream_t stream);
 
+// RMS norm in groups: a row of `width` values is cut into `groups` equal runs, each divided by sqrt(mean(run^2) + eps),
+// the whole times w; x and out fp32 or bf16, sums in fp32. rows: out[r] = norm(x[rows[r]]). gate_kind 1: the row is
+// multiplied by silu(gate[r]) before the norm; 2: the result is multiplied by sigmoid(gate[r]) (no rows then).
+int hfa_group_rmsnorm(const void* x, int x_dtype, int ldx, const float* w, void* out, int out_dtype, int ldo, const int* rows,
+                      int n_rows, int width, int groups, float eps, const void* gate, int gate_dtype, int ldg, int gate_kind,
+                      hipStream_t stream);
+
+// Rows [q: H D | k: G D | v: G Dv] of a step: optional RMS norm of the whole q part and of the whole k part (weights
+// q_norm_w, k_norm_w, eps), rotation of the first rot_dim dimensions of each q and k head (pairing 0: i with i + rot_dim / 2,
+// 1: 2 i with 2 i + 1), optional v <- (1 - *v_blend) v + *v_blend v_other[t] (v_other [T, G Dv]); v_keep [T, G Dv] receives
+// the values as projected. q goes back into the row, k and v into cache rows slot_map[t] (or the row, if null).
+int hfa_qkv_prepare(void* qkv, int dtype, int ld, const int* positions, const float* inv_freq, int rot_dim, int pairing,
+                    int n_heads, int n_kv_heads, int head_dim, int v_head_dim, const float* q_norm_w, const float* k_norm_w,
+                    float eps, const float* v_blend, const void* v_other, void* v_keep, void* k_cache, void* v_cache,
+                    const int* slot_map, int page_tokens, int n_tokens, hipStream_t stream);
+
+// Mixers with per-request state (recurrent.hip). A request's tokens of a step are rows q_start[s] .. q_start[s + 1] - 1;
+// its state is row seq_slot[s] of `state` (fp32, state_ld floats a row).
+// hfa_causal_conv: out[t, c] = act(bias[c] + sum_j taps[c, j] in[t - (K - 1) + j, c]) (fp32 out; act HFA_ACT_SILU or none);
+// inputs before the step's first token come from the state row ([K - 1][C], oldest first), which then receives the
+// step's last K - 1 inputs.
+// hfa_linear_scan: per head h (keys and queries of head h / (n_heads / qk_heads)), S [qk_dim][v_dim] in the state row:
+// S <- a_t S + k_t (b_t v_t)^T, y_t = S^T q_t + skip[h] v_t (skip null: 0). gate 0: a_t = decay[h], b_t = 1. gate 1:
+// dt = softplus(step[t, h] + step_bias[h]), a_t = exp(-exp(a_log[h]) dt), b_t = dt. y fp32.
+int hfa_causal_conv(const void* in, int dtype, int ld_in, const float* taps, const float* bias, int n_channels, int n_taps,
+                    float* state, size_t state_ld, const int* q_start, const int* seq_slot, int n_seqs, int max_q_len, float* out,
+                    int ldo, int act, hipStream_t stream);
+int hfa_linear_scan(const void* q, int ldq, const void* k, int ldk, int qk_heads, int qk_dim, const void* v, int ldv, int n_heads,
+                    int v_dim, int dtype, int gate, const float* decay, const void* step, int step_dtype, int ld_step,
+                    const float* step_bias, const float* a_log, const float* skip, float* state, size_t state_ld,
+                    const int* q_start, const int* seq_slot, int n_seqs, float* y, int ldy, hipStream_t stream);
+
 // out[r, c] = act(in[r, c]) for rows of `width` values with strides ldi and ldo, computed in fp32:
-// the exact gelu 0.5 z (1 + erf(z / sqrt 2)), its tanh form, or relu(z)^2.
+// the exact gelu 0.5 z (1 + erf(z / sqrt 2)), its tanh form, relu(z)^2, silu or the logistic function.
 #ifndef HFA_ACT_GELU_ERF
 #define HFA_ACT_NONE 0
 #define HFA_ACT_GELU_ERF 1
 #define HFA_ACT_GELU_TANH 2
 #define HFA_ACT_RELU2 3
+#define HFA_ACT_SILU 4
+#define HFA_ACT_SIGMOID 5
+#define HFA_ACT_LAST 5
 #endif
 int hfa_activation(const void* in, int ldi, void* out, int ldo, int dtype, int n_rows, int width, int kind,
                    hipStream_t stream);
@@ -158,6 +194,10 @@ int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const void* w, in
                  const int* n_tiles, int max_tiles, int tile_rows, void* out, int ldo, int out_dtype, int out_by_pair,
                  const float* pair_scale, int act, int N, int K, int force_plain, hipStream_t stream);
 int hfa_moe_combine(const float* y, float* x, int n_tokens, int top, int width, hipStream_t stream);
+// Gated experts: row r of the expert-ordered rows holds [gate: F | up: F] fp32 sums; with c = pair_scale[row_pair[r]]
+// (null: 1), g = min(c gate, limit), u = clamp(c up, -limit, limit) (limit <= 0: unbounded): out[r, f] = g sigmoid(alpha g) (u + shift).
+int hfa_moe_gated_act(const float* gu, int ld, const int* row_pair, const float* pair_scale, void* out, int out_dtype, int ldo,
+                      int n_rows, int F, float alpha, float limit, float shift, hipStream_t stream);
 
 // out[t, i] = silu(gate_up[t, i]) * gate_up[t, width + i].  (src/model.c:532-538)
 int hfa_swiglu(const void* gate_up, void* out, int dtype, int n_tokens, int width, hipStream_t stream);

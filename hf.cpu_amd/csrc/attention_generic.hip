@@ -47,7 +47,7 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
     const T* __restrict__ q, int ldq, const T* __restrict__ kc, const T* __restrict__ vc, int kvw, int vw,
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, T* __restrict__ out, int ldo, int H, int G, int D, int Dv, int page_tokens,
-    int window, int mask_chunk, float scale, const float* __restrict__ slopes) {
+    int window, int mask_chunk, float scale, const float* __restrict__ slopes, int sink) {
     __shared__ float q_s[ATT_MAX_D];
     __shared__ float p_s[WAVE];
     __shared__ int row_s[WAVE];
@@ -101,7 +101,7 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
         }
         __syncthreads();
     }
-    const float inv = 1.0f / l;
+    const float inv = 1.0f / (sink ? l + expf(-m) : l);      // the term of score 0 that has no value
 #pragma unroll
     for (int i = 0; i < ATT_MAX_D / WAVE; i++) {
         const int d = lane + WAVE * i;
@@ -112,7 +112,7 @@ __global__ __launch_bounds__(WAVE) void attn_generic_kernel(
 int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache, int kv_width,
                         int v_width, const int* block_table, int max_blocks, const int* token_slot, const int* positions,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
-                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, hipStream_t stream) {
+                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, hipStream_t stream) {
     HFA_REQUIRE(head_dim <= ATT_MAX_D && v_head_dim <= ATT_MAX_D, "paged_attention: head_dim %d (values: %d) exceeds the kernel's limit %d",
                 head_dim, v_head_dim, ATT_MAX_D);
     HFA_REQUIRE(n_heads <= 65535, "paged_attention: %d heads exceed the grid", n_heads);
@@ -120,11 +120,11 @@ int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, 
     if (dtype == HFA_F32)
         attn_generic_kernel<float><<<grid, WAVE, 0, stream>>>(
             (const float*)q, ldq, (const float*)k_cache, (const float*)v_cache, kv_width, v_width, block_table, max_blocks,
-            token_slot, positions, (float*)out, ldo, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window, mask_chunk, scale, slopes);
+            token_slot, positions, (float*)out, ldo, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window, mask_chunk, scale, slopes, sink);
     else
         attn_generic_kernel<bf16><<<grid, WAVE, 0, stream>>>(
             (const bf16*)q, ldq, (const bf16*)k_cache, (const bf16*)v_cache, kv_width, v_width, block_table, max_blocks,
-            token_slot, positions, (bf16*)out, ldo, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window, mask_chunk, scale, slopes);
+            token_slot, positions, (bf16*)out, ldo, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window, mask_chunk, scale, slopes, sink);
     HFA_LAUNCH_CHECK("paged_attention");
     return 0;
 }
@@ -180,7 +180,7 @@ extern "C" int hfa_decode_attention(const float* raw, int ld_raw, const float* c
                 "decode_attention: a row stride is smaller than its row");
     AttnArgs a = {nullptr, 8, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot, positions, q_start,
                   n_seqs, 1, max_seq_len, out, ldo, n_seqs, n_heads, n_kv_heads, head_dim, page_tokens,
-                  window, scale, workspace, workspace_bytes, stream, raw, ld_raw, cos_sin, slot_map, mask_chunk};
+                  window, scale, workspace, workspace_bytes, stream, raw, ld_raw, cos_sin, slot_map, mask_chunk, 0};
     HFA_REQUIRE(((uintptr_t)raw & 15) == 0 && (cos_sin == nullptr || ((uintptr_t)cos_sin & 15) == 0) && attn_mfma_supports(a),
                 "decode_attention: this shape is not taken (see hfa_decode_attention_supports)");
     return attn_mfma_launch(a);
@@ -191,7 +191,7 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
                                    const int* positions, const int* q_start, int n_seqs, int max_q_len,
                                    int max_seq_len, void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads,
                                    int head_dim, int v_head_dim, int page_tokens, int window, int mask_chunk, float scale,
-                                   const float* slopes, void* workspace, size_t workspace_bytes, int force_plain,
+                                   const float* slopes, int sink, void* workspace, size_t workspace_bytes, int force_plain,
                                    hipStream_t stream) {
     HFA_REQUIRE(n_tokens > 0 && n_heads > 0 && n_kv_heads > 0 && head_dim > 0 && v_head_dim > 0 && page_tokens > 0 && max_blocks > 0,
                 "paged_attention: bad sizes");
@@ -204,12 +204,12 @@ extern "C" int hfa_paged_attention(const void* q, int dtype, int ldq, const void
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "paged_attention: unknown dtype %d", dtype);
     AttnArgs a = {q, ldq, k_cache, v_cache, kv_width, block_table, max_blocks, token_slot, positions, q_start,
                   n_seqs, max_q_len, max_seq_len, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, page_tokens,
-                  window, scale, workspace, workspace_bytes, stream, nullptr, 0, nullptr, nullptr, mask_chunk};
+                  window, scale, workspace, workspace_bytes, stream, nullptr, 0, nullptr, nullptr, mask_chunk, sink ? 1 : 0};
     // the matrix-core kernels take no slopes: scores with a position term go the plain way
     // and they know one head size and one row width for keys and values
     if (!force_plain && !slopes && dtype == HFA_BF16 && v_head_dim == head_dim && v_width == kv_width && attn_mfma_supports(a))
         return attn_mfma_launch(a);
     return attn_generic_launch(q, dtype, ldq, k_cache, v_cache, kv_width, v_width, block_table, max_blocks, token_slot,
                                positions, out, ldo, n_tokens, n_heads, n_kv_heads, head_dim, v_head_dim, page_tokens, window,
-                               mask_chunk, scale, slopes, stream);
+                               mask_chunk, scale, slopes, sink ? 1 : 0, stream);
 }

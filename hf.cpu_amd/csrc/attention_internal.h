@@ -19,6 +19,7 @@ struct AttnArgs {
     const float* cos_sin;          // [token][head_dim / 2 cosines, head_dim / 2 sines], null: no rotation
     const int* slot_map;           // the cache row of each token's key and value
     int mask_chunk;                // > 0: a query sees only the keys of its own run of mask_chunk positions, counted from 0
+    int sink;                      // 1: the softmax's denominator holds one more term of score 0 that has no value
 };
 
 // The first key that the query at `pos` sees: a window of the last `window` positions (0: none) and/or the start
@@ -35,7 +36,7 @@ __host__ __device__ __forceinline__ int first_visible(int pos, int window, int m
 int attn_generic_launch(const void* q, int dtype, int ldq, const void* k_cache, const void* v_cache, int kv_width,
                         int v_width, const int* block_table, int max_blocks, const int* token_slot, const int* positions,
                         void* out, int ldo, int n_tokens, int n_heads, int n_kv_heads, int head_dim, int v_head_dim,
-                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, hipStream_t stream);
+                        int page_tokens, int window, int mask_chunk, float scale, const float* slopes, int sink, hipStream_t stream);
 
 // bf16 on the matrix cores; see attention_mfma.hip for what it needs.
 bool attn_mfma_supports(const AttnArgs& a);

@@ -78,7 +78,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
     int ldo, float* __restrict__ partial, int H, int psh, int window, int mask_chunk, float scale_log2e, int tpt, int cpt,
     int chunk_keys, int n_chunks, int one_tile_each, const float* __restrict__ raw, int ld_raw,
-    const float* __restrict__ cs, const int* __restrict__ slot_map, int G) {
+    const float* __restrict__ cs, const int* __restrict__ slot_map, int G, int sink) {
     constexpr int D = NDB * 32, KS = D / 16;
     const int P = 1 << psh;                                // tokens per page, a power of two
     const int lane = threadIdx.x, col = lane & 31, half = lane >> 5;
@@ -454,7 +454,7 @@ __global__ __launch_bounds__(WAVE) void attn_mfma_kernel(
                 *reinterpret_cast<float4*>(dst + 2 + 32 * db + 8 * rg + 4 * half) = v;
             }
     } else {
-        const float inv = 1.0f / l;
+        const float inv = 1.0f / (sink ? l + exp2f(-m) : l);      // the term of score 0 and no value: 2^(0 - m)
         uint16_t* dst = out + (size_t)my_tok * ldo + my_head * D;
 #pragma unroll
         for (int db = 0; db < NDB; db++)
@@ -485,7 +485,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
     const int* __restrict__ block_table, int max_blocks, const int* __restrict__ token_slot,
     const int* __restrict__ positions, const int* __restrict__ q_start, int n_seqs, uint16_t* __restrict__ out,
     int ldo, int psh, int window, int mask_chunk, float scale_log2e, int tpt, int cpt, int n_tiles, int pair_from,
-    float* __restrict__ partial, int H, int chunk_keys, int n_chunks) {
+    float* __restrict__ partial, int H, int chunk_keys, int n_chunks, int sink) {
     constexpr int D = NDB * 32, KS = D / 16, KROW = D + 8;
     const int P = 1 << psh;                                // tokens per page, a power of two
     __shared__ __attribute__((aligned(16))) uint16_t k_s[2][KB * KROW];
@@ -794,7 +794,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
                     make_float4(o[db][4 * rg], o[db][4 * rg + 1], o[db][4 * rg + 2], o[db][4 * rg + 3]);
         return;
     }
-    const float inv = 1.0f / l;
+    const float inv = 1.0f / (sink ? l + exp2f(-m) : l);          // the term of score 0 and no value: 2^(0 - m)
     uint16_t* dst = out + (size_t)my_tok * ldo + my_head * D;
 #pragma unroll
     for (int db = 0; db < NDB; db++)
@@ -815,7 +815,7 @@ __global__ __launch_bounds__(4 * WAVE) __attribute__((amdgpu_waves_per_eu(2))) v
 #define MERGE_MAX_CHUNKS 512
 #define MERGE_GROUP 16
 __global__ __launch_bounds__(WAVE) void attn_merge_kernel(const float* __restrict__ partial, uint16_t* __restrict__ out,
-                                                          int ldo, int H, int D, int n_chunks) {
+                                                          int ldo, int H, int D, int n_chunks, int sink) {
     __shared__ float w_s[MERGE_MAX_CHUNKS];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const size_t row = D + 2;
@@ -843,6 +843,7 @@ __global__ __launch_bounds__(WAVE) void attn_merge_kernel(const float* __restric
         L += ml.y * w;
     }
     L = wave_sum(L);
+    if (sink) L += exp2f(-M);                            // once for all chunks: the term of score 0 and no value
     __syncthreads();
     if (!has) return;
     float ax = 0.f, ay = 0.f;
@@ -893,7 +894,7 @@ static int launch_ndb(const AttnArgs& a, int tiles, int tpt, int cpt, int chunk_
     (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,      \
         a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo, PARTIAL, a.n_heads,         \
         page_shift(a.page_tokens), a.window, a.mask_chunk, sl, tpt, cpt, chunk_keys, n_chunks, a.max_q_len <= tpt, a.raw, a.ld_raw,      \
-        a.cos_sin, a.slot_map, a.n_kv_heads
+        a.cos_sin, a.slot_map, a.n_kv_heads, a.sink
     if (a.raw) {
         if (n_chunks > 1) attn_mfma_kernel<NDB, true, true><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS((float*)a.workspace));
         else attn_mfma_kernel<NDB, false, true><<<grid, WAVE, 0, a.stream>>>(ATTN_ARGS(nullptr));
@@ -953,17 +954,17 @@ static int launch_prefill(const AttnArgs& a, int tpt, int cpt) {
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
             a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
             page_shift(a.page_tokens), a.window, a.mask_chunk, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
-            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks);
+            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks, a.sink);
     else
         attn_prefill_kernel<NDB, false><<<grid, 4 * WAVE, 0, a.stream>>>(
             (const uint16_t*)a.q, a.ldq, (const uint16_t*)a.k_cache, (const uint16_t*)a.v_cache, a.kv_width, a.block_table,
             a.max_blocks, a.token_slot, a.positions, a.q_start, a.n_seqs, (uint16_t*)a.out, a.ldo,
             page_shift(a.page_tokens), a.window, a.mask_chunk, a.scale * 1.4426950408889634f, tpt, cpt, n_tiles, pair_from,
-            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks);
+            (float*)a.workspace, a.n_heads, chunk_keys, n_chunks, a.sink);
     HFA_LAUNCH_CHECK("attn_prefill");
     if (n_chunks > 1) {
         attn_merge_kernel<<<dim3(a.n_tokens, a.n_heads), WAVE, 0, a.stream>>>((const float*)a.workspace, (uint16_t*)a.out, a.ldo,
-                                                                            a.n_heads, a.head_dim, n_chunks);
+                                                                            a.n_heads, a.head_dim, n_chunks, a.sink);
         HFA_LAUNCH_CHECK("attn_merge");
     }
     return 0;
@@ -1030,7 +1031,7 @@ int attn_mfma_launch(const AttnArgs& a) {
     if (rc || n_chunks == 1) return rc;
     dim3 grid(a.n_tokens, a.n_heads);
     attn_merge_kernel<<<grid, WAVE, 0, a.stream>>>((const float*)a.workspace, (uint16_t*)a.out, a.ldo, a.n_heads,
-                                                  a.head_dim, n_chunks);
+                                                  a.head_dim, n_chunks, a.sink);
     HFA_LAUNCH_CHECK("attn_merge");
     return 0;
 }

@@ -74,11 +74,16 @@ __device__ __forceinline__ float block_max(float v, float* red) {
 #define HFA_ACT_GELU_ERF 1
 #define HFA_ACT_GELU_TANH 2
 #define HFA_ACT_RELU2 3
+#define HFA_ACT_SILU 4
+#define HFA_ACT_SIGMOID 5
+#define HFA_ACT_LAST 5
 #endif
 __device__ __forceinline__ float hfa_act_apply(int kind, float z) {
     if (kind == HFA_ACT_GELU_ERF) return 0.5f * z * (1.0f + erff(z * 0.70710678118654752f));
     if (kind == HFA_ACT_GELU_TANH) return 0.5f * z * (1.0f + tanhf(0.79788456080286536f * (z + 0.044715f * z * z * z)));
     if (kind == HFA_ACT_RELU2) { const float r = fmaxf(z, 0.f); return r * r; }
+    if (kind == HFA_ACT_SILU) return z / (1.0f + expf(-z));
+    if (kind == HFA_ACT_SIGMOID) return 1.0f / (1.0f + expf(-z));
     return z;
 }
 

@@ -449,3 +449,101 @@ extern "C" int hfa_random_fill(void* out, int dtype, size_t n, uint64_t key, flo
     HFA_LAUNCH_CHECK("random_fill");
     return 0;
 }
+
+// ---- queries and keys normed over the whole projection, rotation in either pairing, blended values, cache store ----
+// One block a token, whose row holds [q: H D | k: G D | v: G Dv]. In this order:
+//   q_norm_w / k_norm_w (fp32 [H D] / [G D], either may be null): the whole q part (k part) is divided by
+//   sqrt(mean of its squares + eps) and multiplied by the weights, before the rotation;
+//   rotation of the first rot_dim dimensions of every q and k head by positions[t] * inv_freq[i]: pairing 0 pairs
+//   dimension i with i + rot_dim / 2, pairing 1 dimension 2 i with 2 i + 1;
+//   v_blend (a scalar on the device) with v_other ([T, G Dv], the values that an earlier layer kept for the same
+//   tokens): v <- (1 - v_blend) v + v_blend v_other;  v_keep ([T, G Dv]) receives this layer's values as projected.
+// q is written back into the row; k and v go to the cache rows slot_map[t] (values transposed inside their page), or
+// back into the row where slot_map is null.
+template <typename T>
+__global__ __launch_bounds__(256) void qkv_prepare_kernel(
+    T* __restrict__ qkv, int ld, const int* __restrict__ positions, const float* __restrict__ inv_freq, int rot_dim,
+    int pairing, int H, int G, int D, int Dv, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w,
+    float eps, const float* __restrict__ v_blend, const T* __restrict__ v_other, T* __restrict__ v_keep,
+    T* __restrict__ k_cache, T* __restrict__ v_cache, const int* __restrict__ slot_map, int page_tokens) {
+    __shared__ float red[17];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    T* row = qkv + (size_t)t * ld;
+    const int QD = H * D, KD = G * D, VD = G * Dv;
+    float q_inv = 1.f, k_inv = 1.f;
+    if (q_norm_w) {
+        float ss = 0.f;
+        for (int i = tid; i < QD; i += blockDim.x) { const float x = to_f32(row[i]); ss = fmaf(x, x, ss); }
+        q_inv = 1.0f / sqrtf(block_sum(ss, red) / (float)QD + eps);
+    }
+    if (k_norm_w) {
+        float ss = 0.f;
+        for (int i = tid; i < KD; i += blockDim.x) { const float x = to_f32(row[QD + i]); ss = fmaf(x, x, ss); }
+        k_inv = 1.0f / sqrtf(block_sum(ss, red) / (float)KD + eps);
+    }
+    const int slot = slot_map ? slot_map[t] : -1;
+    const float pos = rot_dim > 0 ? (float)positions[t] : 0.f;
+    const int half = rot_dim / 2, pairs_per_head = half + (D - rot_dim);      // work items of a head: pairs, then single dimensions
+    // queries and keys: item (head slot hs, j): j < half is the pair j, the rest the dimensions that pass
+    for (int it = tid; it < (H + G) * pairs_per_head; it += blockDim.x) {
+        const int hs = it / pairs_per_head, j = it % pairs_per_head;
+        const bool is_key = hs >= H;
+        const int base = hs * D;                                   // the head's first column in the row (keys follow the queries)
+        const float inv = is_key ? k_inv : q_inv;
+        const float* nw = is_key ? k_norm_w : q_norm_w;
+        const int nbase = is_key ? base - QD : base;
+        T* dst = (is_key && slot >= 0) ? k_cache + (size_t)slot * KD + (hs - H) * D : row + base;
+        if (j < half) {
+            const int i0 = pairing == 1 ? 2 * j : j, i1 = pairing == 1 ? 2 * j + 1 : j + half;
+            float x0 = to_f32(row[base + i0]) * inv, x1 = to_f32(row[base + i1]) * inv;
+            if (nw) { x0 *= nw[nbase + i0]; x1 *= nw[nbase + i1]; }
+            float sn, cs;
+            sincosf(pos * inv_freq[j], &sn, &cs);
+            dst[i0] = from_f32<T>(x0 * cs - x1 * sn);
+            dst[i1] = from_f32<T>(x1 * cs + x0 * sn);
+        } else {
+            const int i = rot_dim + (j - half);
+            float x = to_f32(row[base + i]) * inv;
+            if (nw) x *= nw[nbase + i];
+            dst[i] = from_f32<T>(x);
+        }
+    }
+    const float lam = v_blend ? *v_blend : 0.f;
+    for (int c = tid; c < VD; c += blockDim.x) {
+        float x = to_f32(row[QD + KD + c]);
+        if (v_keep) v_keep[(size_t)t * VD + c] = from_f32<T>(x);
+        if (v_other) x = (1.0f - lam) * x + lam * to_f32(v_other[(size_t)t * VD + c]);
+        if (slot >= 0)
+            v_cache[(size_t)(slot / page_tokens) * page_tokens * VD + (size_t)c * page_tokens + slot % page_tokens] = from_f32<T>(x);
+        else
+            row[QD + KD + c] = from_f32<T>(x);
+    }
+}
+
+extern "C" int hfa_qkv_prepare(void* qkv, int dtype, int ld, const int* positions, const float* inv_freq, int rot_dim,
+                               int pairing, int n_heads, int n_kv_heads, int head_dim, int v_head_dim, const float* q_norm_w,
+                               const float* k_norm_w, float eps, const float* v_blend, const void* v_other, void* v_keep,
+                               void* k_cache, void* v_cache, const int* slot_map, int page_tokens, int n_tokens,
+                               hipStream_t stream) {
+    HFA_REQUIRE(qkv && n_tokens > 0 && n_heads > 0 && n_kv_heads >= 0 && head_dim > 0 && v_head_dim > 0, "qkv_prepare: bad sizes");
+    HFA_REQUIRE(rot_dim >= 0 && rot_dim % 2 == 0 && rot_dim <= head_dim, "qkv_prepare: rot_dim %d must be even and at most head_dim %d",
+                rot_dim, head_dim);
+    HFA_REQUIRE(rot_dim == 0 || (positions && inv_freq), "qkv_prepare: positions and inv_freq are needed");
+    HFA_REQUIRE(pairing == 0 || pairing == 1, "qkv_prepare: pairing %d is neither 0 (halves) nor 1 (neighbours)", pairing);
+    HFA_REQUIRE(ld >= (n_heads + n_kv_heads) * head_dim + n_kv_heads * v_head_dim, "qkv_prepare: row stride %d is too small", ld);
+    HFA_REQUIRE(!slot_map || (k_cache && v_cache && page_tokens > 0 && n_kv_heads > 0), "qkv_prepare: no cache to store into");
+    HFA_REQUIRE((!v_blend && !v_other) || (v_blend && v_other && n_kv_heads > 0), "qkv_prepare: blending needs the weight and the other values");
+    HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "qkv_prepare: unknown dtype %d", dtype);
+    if (dtype == HFA_F32)
+        qkv_prepare_kernel<float><<<n_tokens, 256, 0, stream>>>((float*)qkv, ld, positions, inv_freq, rot_dim, pairing, n_heads,
+                                                                n_kv_heads, head_dim, v_head_dim, q_norm_w, k_norm_w, eps, v_blend,
+                                                                (const float*)v_other, (float*)v_keep, (float*)k_cache,
+                                                                (float*)v_cache, slot_map, page_tokens);
+    else
+        qkv_prepare_kernel<bf16><<<n_tokens, 256, 0, stream>>>((bf16*)qkv, ld, positions, inv_freq, rot_dim, pairing, n_heads,
+                                                               n_kv_heads, head_dim, v_head_dim, q_norm_w, k_norm_w, eps, v_blend,
+                                                               (const bf16*)v_other, (bf16*)v_keep, (bf16*)k_cache, (bf16*)v_cache,
+                                                               slot_map, page_tokens);
+    HFA_LAUNCH_CHECK("qkv_prepare");
+    return 0;
+}

@@ -14,7 +14,7 @@ extern "C" int hfa_gemm(const void* a, int a_dtype, int lda, const void* w, int 
                     (out_dtype == HFA_F32 || out_dtype == HFA_BF16),
                 "gemm: unknown dtype (a=%d w=%d out=%d)", a_dtype, w_dtype, out_dtype);
     HFA_REQUIRE(!accumulate || out_dtype == HFA_F32, "gemm: accumulation needs an fp32 output");
-    HFA_REQUIRE(epilogue >= 0 && epilogue <= 1 + HFA_ACT_RELU2, "gemm: unknown epilogue %d", epilogue);
+    HFA_REQUIRE(epilogue >= 0 && epilogue <= 1 + HFA_ACT_LAST, "gemm: unknown epilogue %d", epilogue);
     const int act = epilogue >= 2 ? epilogue - 1 : 0;
     HFA_REQUIRE(!act || !accumulate, "gemm: an activation goes with a plain output, not with accumulation");
     if (act) {

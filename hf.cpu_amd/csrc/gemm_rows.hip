@@ -463,7 +463,7 @@ extern "C" int hfa_gemm_rows(int mode, const void* a, int lda, const void* w, in
     p.bias = bias; p.ssq_in = ssq_in; p.parts_in = parts_in; p.inv_width = inv_width; p.eps = eps;
     if (mode == HFA_ROWS_OUT) {
         HFA_REQUIRE(out && ldo >= N && (out_dtype == HFA_F32 || out_dtype == HFA_BF16), "gemm_rows: no output, or its rows are shorter than N");
-        HFA_REQUIRE(out_act >= 0 && out_act <= HFA_ACT_RELU2, "gemm_rows: unknown activation %d", out_act);
+        HFA_REQUIRE(out_act >= 0 && out_act <= HFA_ACT_LAST, "gemm_rows: unknown activation %d", out_act);
         p.out = out; p.ldo = ldo; p.out_bf16 = out_dtype == HFA_BF16; p.out_act = out_act;
         return rows_dispatch<HFA_ROWS_OUT>(p, stream);
     }

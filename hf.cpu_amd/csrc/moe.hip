@@ -494,7 +494,7 @@ extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const 
                 "moe_gemm: bad arguments");
     HFA_REQUIRE((dtype == HFA_F32 || dtype == HFA_BF16) && (out_dtype == HFA_F32 || out_dtype == HFA_BF16) &&
                     (w_dtype == HFA_F32 || w_dtype == HFA_BF16), "moe_gemm: unknown dtype");
-    HFA_REQUIRE(act >= 0 && act <= HFA_ACT_RELU2 && a_div >= 0, "moe_gemm: bad activation or divisor");
+    HFA_REQUIRE(act >= 0 && act <= HFA_ACT_LAST && a_div >= 0, "moe_gemm: bad activation or divisor");
     const bool mfma = !force_plain && dtype == HFA_BF16 && w_dtype == HFA_BF16 && K % 16 == 0 && N % 32 == 0 && lda % 8 == 0 &&
                       (tile_rows == 32 || tile_rows == 64 || tile_rows == 128) && ((uintptr_t)a & 15) == 0 && ((uintptr_t)w & 15) == 0;
     if (mfma && tile_rows >= 64) {
@@ -594,5 +594,40 @@ extern "C" int hfa_moe_combine(const float* y, float* x, int n_tokens, int top, 
     if (vec) moe_combine4_kernel<<<blocks, 256, 0, stream>>>((const float4*)y, (float4*)x, top, width / 4, total);
     else moe_combine_kernel<<<blocks, 256, 0, stream>>>(y, x, top, width, total);
     HFA_LAUNCH_CHECK("moe_combine");
+    return 0;
+}
+
+// ---- gated experts ------------------------------------------------------------------------
+// Row r of the expert-ordered rows holds [gate: F | up: F] fp32 sums of one (token, choice) pair. With c = pair_scale of
+// the row's pair (null: 1), g = min(c gate, limit), u = clamp(c up, -limit, limit) (limit <= 0: no bounds):
+// mid[r, f] = g sigmoid(alpha g) (u + shift). Scaling the sums is scaling the expert's input.
+template <typename TO>
+__global__ void moe_gated_act_kernel(const float* __restrict__ gu, int ld, const int* __restrict__ row_pair,
+                                     const float* __restrict__ pair_scale, TO* __restrict__ out, int ldo, int F, float alpha,
+                                     float limit, float shift, size_t total) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
+        const size_t r = i / F, f = i % F;
+        const float c = pair_scale ? pair_scale[row_pair[r]] : 1.f;
+        float g = c * gu[r * ld + f], u = c * gu[r * ld + F + f];
+        if (limit > 0.f) {
+            g = fminf(g, limit);
+            u = fminf(fmaxf(u, -limit), limit);
+        }
+        out[r * ldo + f] = from_f32<TO>(g / (1.0f + expf(-alpha * g)) * (u + shift));
+    }
+}
+
+extern "C" int hfa_moe_gated_act(const float* gu, int ld, const int* row_pair, const float* pair_scale, void* out,
+                                 int out_dtype, int ldo, int n_rows, int F, float alpha, float limit, float shift,
+                                 hipStream_t stream) {
+    HFA_REQUIRE(gu && out && n_rows > 0 && F > 0 && ld >= 2 * F && ldo >= F && (!pair_scale || row_pair), "moe_gated_act: bad arguments");
+    HFA_REQUIRE(out_dtype == HFA_F32 || out_dtype == HFA_BF16, "moe_gated_act: unknown dtype %d", out_dtype);
+    const size_t total = (size_t)n_rows * F;
+    const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
+    if (out_dtype == HFA_F32)
+        moe_gated_act_kernel<float><<<blocks, 256, 0, stream>>>(gu, ld, row_pair, pair_scale, (float*)out, ldo, F, alpha, limit, shift, total);
+    else
+        moe_gated_act_kernel<bf16><<<blocks, 256, 0, stream>>>(gu, ld, row_pair, pair_scale, (bf16*)out, ldo, F, alpha, limit, shift, total);
+    HFA_LAUNCH_CHECK("moe_gated_act");
     return 0;
 }

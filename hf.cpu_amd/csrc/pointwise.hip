@@ -1,4 +1,4 @@
-// Layer norm with scale and shift, the activations of the plain feed-forward layers (erf gelu, tanh gelu,
+// Layer norm with scale and shift, the RMS norm in groups (with a gate), the activations of the plain feed-forward layers (erf gelu, tanh gelu,
 // squared relu) and the soft cap of the logits.
 #include "api.h"
 #include "common.h"
@@ -101,7 +101,7 @@ __global__ void activation_kernel(const T* __restrict__ in, int ldi, T* __restri
 extern "C" int hfa_activation(const void* in, int ldi, void* out, int ldo, int dtype, int n_rows, int width, int kind,
                               hipStream_t stream) {
     HFA_REQUIRE(in && out && n_rows > 0 && width > 0 && ldi >= width && ldo >= width, "activation: bad arguments");
-    HFA_REQUIRE(kind >= HFA_ACT_GELU_ERF && kind <= HFA_ACT_RELU2, "activation: unknown kind %d", kind);
+    HFA_REQUIRE(kind >= HFA_ACT_GELU_ERF && kind <= HFA_ACT_LAST, "activation: unknown kind %d", kind);
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "activation: unknown dtype %d", dtype);
     const size_t total = (size_t)n_rows * width;
     const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
@@ -128,5 +128,81 @@ extern "C" int hfa_softcap(float* x, int ld, int n_rows, int width, float cap, h
     const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
     softcap_kernel<<<blocks, 256, 0, stream>>>(x, ld, width, cap, 1.0f / cap, total);
     HFA_LAUNCH_CHECK("softcap");
+    return 0;
+}
+
+// ---- RMS norm in groups, with an optional gate ----------------------------------------------
+// A row of `width` values is cut into `groups` equal runs; each run is divided by sqrt(mean(run^2) + eps) and the
+// whole is multiplied by w (one block a (row, run); sums in fp32 in a fixed order). gate_kind 1: the row is first
+// multiplied by silu(gate) (the gate comes before the norm); gate_kind 2: the normed and weighted row is multiplied
+// by sigmoid(gate) (the gate comes after). `rows`: out[r] is the norm of x[rows[r]] (the gate's rows are not gathered).
+template <typename TX, typename TG, typename TO>
+__global__ __launch_bounds__(1024) void group_rmsnorm_kernel(const TX* __restrict__ x, int ldx, const float* __restrict__ w,
+                                                            TO* __restrict__ out, int ldo, const int* __restrict__ rows,
+                                                            int run, float eps, const TG* __restrict__ gate, int ldg,
+                                                            int gate_kind) {
+    __shared__ float red[17];
+    const int r = blockIdx.x, c0 = blockIdx.y * run;
+    const TX* src = x + (size_t)(rows ? rows[r] : r) * ldx + c0;
+    const TG* gsrc = gate ? gate + (size_t)r * ldg + c0 : nullptr;
+    constexpr int KEEP = 4;
+    float keep[KEEP];
+    auto value = [&](int i) {
+        float v = to_f32(src[i]);
+        if (gate_kind == 1) {
+            const float z = to_f32(gsrc[i]);
+            v *= z / (1.0f + expf(-z));
+        }
+        return v;
+    };
+    float ss = 0.f;
+#pragma unroll
+    for (int k = 0; k < KEEP; k++) {
+        const int i = threadIdx.x + k * blockDim.x;
+        keep[k] = i < run ? value(i) : 0.f;
+        ss = fmaf(keep[k], keep[k], ss);
+    }
+    for (int i = threadIdx.x + KEEP * blockDim.x; i < run; i += blockDim.x) {
+        const float v = value(i);
+        ss = fmaf(v, v, ss);
+    }
+    const float inv = 1.0f / sqrtf(block_sum(ss, red) / (float)run + eps);
+    TO* dst = out + (size_t)r * ldo + c0;
+    auto finish = [&](int i, float v) {
+        float y = v * inv * w[c0 + i];
+        if (gate_kind == 2) y *= 1.0f / (1.0f + expf(-to_f32(gsrc[i])));
+        dst[i] = from_f32<TO>(y);
+    };
+#pragma unroll
+    for (int k = 0; k < KEEP; k++) {
+        const int i = threadIdx.x + k * blockDim.x;
+        if (i < run) finish(i, keep[k]);
+    }
+    for (int i = threadIdx.x + KEEP * blockDim.x; i < run; i += blockDim.x) finish(i, value(i));
+}
+
+extern "C" int hfa_group_rmsnorm(const void* x, int x_dtype, int ldx, const float* w, void* out, int out_dtype, int ldo,
+                                 const int* rows, int n_rows, int width, int groups, float eps, const void* gate,
+                                 int gate_dtype, int ldg, int gate_kind, hipStream_t stream) {
+    HFA_REQUIRE(x && w && out && n_rows > 0 && width > 0 && ldx >= width && ldo >= width, "group_rmsnorm: bad arguments");
+    HFA_REQUIRE(groups > 0 && width % groups == 0 && groups <= 65535, "group_rmsnorm: %d values do not form %d equal runs", width, groups);
+    HFA_REQUIRE((x_dtype == HFA_F32 || x_dtype == HFA_BF16) && (out_dtype == HFA_F32 || out_dtype == HFA_BF16),
+                "group_rmsnorm: unknown dtype");
+    HFA_REQUIRE(gate_kind >= 0 && gate_kind <= 2 && (gate_kind == 0 || (gate && ldg >= width && !rows &&
+                                                                       (gate_dtype == HFA_F32 || gate_dtype == HFA_BF16))),
+                "group_rmsnorm: a gate needs its rows, one for each row in order");
+    const int run = width / groups;
+    const int threads = run >= 4096 ? 1024 : run >= 1024 ? 256 : run >= 256 ? 128 : 64;
+    dim3 grid(n_rows, groups);
+#define GRN(TX, TG, TO)                                                                                                 \
+    group_rmsnorm_kernel<TX, TG, TO><<<grid, threads, 0, stream>>>((const TX*)x, ldx, w, (TO*)out, ldo, rows, run, eps, \
+                                                                   (const TG*)(gate_kind ? gate : nullptr), ldg, gate_kind)
+    const bool gb = gate_kind && gate_dtype == HFA_BF16;
+    if (x_dtype == HFA_F32 && out_dtype == HFA_F32) { if (gb) GRN(float, bf16, float); else GRN(float, float, float); }
+    else if (x_dtype == HFA_F32) { if (gb) GRN(float, bf16, bf16); else GRN(float, float, bf16); }
+    else if (out_dtype == HFA_F32) { if (gb) GRN(bf16, bf16, float); else GRN(bf16, float, float); }
+    else { if (gb) GRN(bf16, bf16, bf16); else GRN(bf16, float, bf16); }
+#undef GRN
+    HFA_LAUNCH_CHECK("group_rmsnorm");
     return 0;
 }

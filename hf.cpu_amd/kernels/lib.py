@@ -21,7 +21,12 @@ _SIGNATURES = {
     "hfa_gemm_rows": [I, P, I, P, I, I, I, I, P, P, I, F, F, P, I, I, I, P, I, P, P, P, I, P, I, P],
     "hfa_gemm_rows_supports": [I, I, I, I, I, I],
     "hfa_rope_store": [P, I, I, P, P, I, I, I, I, I, P, P, P, I, I, P, I, P, P],
-    "hfa_paged_attention": [P, I, I, P, P, I, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, I, F, P, P, c_size_t, I, P],
+    "hfa_paged_attention": [P, I, I, P, P, I, I, P, I, P, P, P, I, I, I, P, I, I, I, I, I, I, I, I, I, F, P, I, P, c_size_t, I, P],
+    "hfa_group_rmsnorm": [P, I, I, P, P, I, I, P, I, I, I, F, P, I, I, I, P],
+    "hfa_qkv_prepare": [P, I, I, P, P, I, I, I, I, I, I, P, P, F, P, P, P, P, P, P, I, I, P],
+    "hfa_causal_conv": [P, I, I, P, P, I, I, P, c_size_t, P, P, I, I, P, I, I, P],
+    "hfa_linear_scan": [P, I, P, I, I, I, P, I, I, I, I, I, P, P, I, I, P, P, P, P, c_size_t, P, P, I, P, I, P],
+    "hfa_moe_gated_act": [P, I, P, P, P, I, I, I, I, F, F, F, P],
     "hfa_rope_table": [P, P, I, P, I, P],
     "hfa_decode_attention_supports": [I, I, I, I, I, I, I, I],
     "hfa_decode_attention": [P, I, P, P, P, I, P, P, I, P, P, P, I, I, P, I, I, I, I, I, I, I, F, P, c_size_t, P],

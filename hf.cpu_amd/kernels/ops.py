@@ -525,17 +525,18 @@ class Ops:
             None if pend is None or pend.bias is None else pend.bias.data_ptr(), self._stream()))
 
     def paged_attention(self, q, n_heads, n_kv_heads, head_dim, cache, step, window, scale, out, slopes=None,
-                        v_head_dim=None, mask_chunk=0):
+                        v_head_dim=None, mask_chunk=0, sink=False):
         """Attention of the first ``n_heads * head_dim`` columns of ``q`` over ``cache``. ``slopes``
         (fp32, one per query head): the score of key j for the query at p gets ``slopes[h] * (j - p)``
         added, for position encodings that enter the scores; the plain kernel then runs, as it does when
         value heads have a size of their own (``v_head_dim``; ``out`` then has that many columns a head).
-        ``mask_chunk`` > 0: a query sees only the keys of its own run of that many positions, counted from 0."""
+        ``mask_chunk`` > 0: a query sees only the keys of its own run of that many positions, counted from 0.
+        ``sink``: the softmax's denominator holds one more term of score 0 that has no value."""
         v_head_dim = head_dim if v_head_dim is None else int(v_head_dim)
         mask_chunk = int(mask_chunk)
         self._scaled.pop(out.data_ptr(), None)               # whatever `out` held, it is no norm's lazy output any more
         lr = self._lazy_rope
-        if lr is not None and lr.qkv.data_ptr() == q.data_ptr() and lr.cache is cache and slopes is None \
+        if lr is not None and lr.qkv.data_ptr() == q.data_ptr() and lr.cache is cache and slopes is None and not sink \
                 and step.max_q_len == 1 and step.n_seqs == q.shape[0] and not self.force_plain_attention \
                 and out.dtype == torch.bfloat16 and v_head_dim == head_dim and lr.args[4] == n_heads and lr.args[6] == head_dim \
                 and lr.args[5] in (0, n_kv_heads) and cache.k.shape[1] == n_kv_heads * head_dim \
@@ -571,7 +572,7 @@ class Ops:
                 step.token_slot.data_ptr() + 4 * first, step.positions.data_ptr() + 4 * first, q_start.data_ptr(), n_seqs,
                 max_q_len, step.max_seq_len, out.data_ptr() + first * ldo * out.element_size(), ldo, n_tokens, n_heads,
                 n_kv_heads, head_dim, v_head_dim, cache.page_tokens, int(window), mask_chunk, float(scale),
-                None if slopes is None else slopes.data_ptr(), self.attn_workspace.data_ptr(),
+                None if slopes is None else slopes.data_ptr(), 1 if sink else 0, self.attn_workspace.data_ptr(),
                 self.attn_workspace.numel(), 1 if plain else 0, self._stream()))
 
         # Decoded tokens beside prompt portions: one call would send all of them to the kernel for prompt
@@ -623,6 +624,123 @@ class Ops:
             fail(EINVAL, "swiglu: expected contiguous [T, 2F] in and [T, F] out of one dtype")
         self._check(self.lib.hfa_swiglu(gate_up.data_ptr(), out.data_ptr(), _code(out), T, F2 // 2, self._stream()))
 
+    # ---- norms in groups, queries and keys normed whole, mixers with per-request state -------------------------------
+    GATES = {None: 0, "silu_before": 1, "sigmoid_after": 2}
+
+    def group_rmsnorm(self, x, weight, eps, groups, out, rows=None, gate=None, gate_kind=None):
+        """``out[r] = norm(x[rows[r]])``: the row is cut into ``groups`` equal runs, each divided by its own root mean
+        square (``eps`` inside the root), the whole times ``weight``; sums in fp32. ``gate`` (a matrix with the rows of
+        ``out``) with ``gate_kind`` ``silu_before`` (the row times silu(gate) is normed) or ``sigmoid_after`` (the normed
+        row is multiplied by sigmoid(gate))."""
+        self.settle()
+        self._whole(x)
+        self._scaled.pop(out.data_ptr(), None)
+        R, E = out.shape
+        if gate_kind not in self.GATES or (gate is None) != (gate_kind is None):
+            fail(EINVAL, f"group_rmsnorm: a gate comes with its kind, one of {', '.join(k for k in self.GATES if k)}")
+        if x.shape[1] != E or weight.dtype != torch.float32 or weight.numel() != E or not weight.is_contiguous() or E % int(groups):
+            fail(EINVAL, f"group_rmsnorm: rows of {x.shape[1]}, {weight.numel()} fp32 weights, rows of {E} out, {groups} equal runs")
+        if rows is None and R != x.shape[0]:
+            fail(EINVAL, "group_rmsnorm: without row indices the output must have x's rows")
+        if gate is not None and (gate.shape[0] != R or gate.shape[1] != E or rows is not None):
+            fail(EINVAL, "group_rmsnorm: the gate has the output's shape, and no rows are gathered with it")
+        self._check(self.lib.hfa_group_rmsnorm(
+            x.data_ptr(), _code(x), _rows(x, "norm in"), weight.data_ptr(), out.data_ptr(), _code(out), _rows(out, "norm out"),
+            None if rows is None else _ints(rows, "norm rows", R), R, E, int(groups), float(eps),
+            None if gate is None else gate.data_ptr(), 0 if gate is None else _code(gate),
+            0 if gate is None else _rows(gate, "norm gate"), self.GATES[gate_kind], self._stream()))
+
+    PAIRINGS = {"split_half": 0, "interleaved": 1}
+
+    def qkv_prepare(self, qkv, positions, inv_freq, rot_dim, pairing, n_heads, n_kv_heads, head_dim, v_head_dim, cache, slot_map,
+                    q_norm=None, k_norm=None, eps=0.0, v_blend=None, v_other=None, v_keep=None):
+        """What lies between the q/k/v product and attention when ``rope_store`` does not do: rows ``[q | k | v]``;
+        ``q_norm`` / ``k_norm`` (fp32 weights over the whole q part / k part): RMS norm of that part before the rotation;
+        rotation of the first ``rot_dim`` dimensions of each head in ``pairing`` (``split_half``: i with i + rot_dim/2;
+        ``interleaved``: 2i with 2i + 1); ``v_blend`` (a scalar on the device) and ``v_other`` ([T, values]):
+        ``v <- (1 - v_blend) v + v_blend v_other``; ``v_keep`` ([T, values]) receives the values as projected. Keys and
+        values go to ``cache`` at ``slot_map`` (values transposed inside their page)."""
+        self.settle()
+        self._whole(qkv)
+        if pairing not in self.PAIRINGS:
+            fail(ENOTSUP, f"rotary pairing '{pairing}' is not one of {', '.join(self.PAIRINGS)}")
+        T = qkv.shape[0]
+        QD, KD, VD = n_heads * head_dim, n_kv_heads * head_dim, n_kv_heads * v_head_dim
+        if qkv.shape[1] < QD + KD + VD:
+            fail(EINVAL, "qkv_prepare: the rows are narrower than the heads they should hold")
+        for w, n, what in ((q_norm, QD, "q_norm"), (k_norm, KD, "k_norm")):
+            if w is not None and (w.dtype != torch.float32 or w.numel() != n or not w.is_contiguous()):
+                fail(EINVAL, f"qkv_prepare: {what} must be {n} contiguous fp32 weights")
+        for t, what in ((v_other, "v_other"), (v_keep, "v_keep")):
+            if t is not None and (t.dtype != qkv.dtype or tuple(t.shape) != (T, VD) or not t.is_contiguous()):
+                fail(EINVAL, f"qkv_prepare: {what} must be [{T}, {VD}] of the rows' dtype")
+        if (v_blend is None) != (v_other is None) or (v_blend is not None and (v_blend.dtype != torch.float32 or v_blend.numel() != 1)):
+            fail(EINVAL, "qkv_prepare: blending needs one fp32 weight on the device and the other values")
+        k_ptr = v_ptr = None
+        if slot_map is not None:
+            for c, width in ((cache.k, KD), (cache.v, VD)):
+                if c.dtype != qkv.dtype or c.dim() != 2 or c.shape[1] != width or not c.is_contiguous():
+                    fail(EINVAL, f"qkv_prepare: the cache must have the activations' dtype and one row of {width} values per token")
+            k_ptr, v_ptr = cache.k.data_ptr(), cache.v.data_ptr()
+
+        def ptr(t):
+            return None if t is None else t.data_ptr()
+        self._check(self.lib.hfa_qkv_prepare(
+            qkv.data_ptr(), _code(qkv), _rows(qkv, "qkv"), None if rot_dim == 0 else _ints(positions, "positions", T),
+            None if rot_dim == 0 else inv_freq.data_ptr(), int(rot_dim), self.PAIRINGS[pairing], n_heads, n_kv_heads, head_dim,
+            v_head_dim, ptr(q_norm), ptr(k_norm), float(eps), ptr(v_blend), ptr(v_other), ptr(v_keep), k_ptr, v_ptr,
+            None if slot_map is None else _ints(slot_map, "slot_map", T), getattr(cache, "page_tokens", 0) or 0, T, self._stream()))
+
+    def causal_conv(self, x, taps, bias, state, step, out, activation=None):
+        """``out[t, c] = act(bias[c] + sum_j taps[c, j] x[t - (K - 1) + j, c])`` along each request's tokens (fp32 out);
+        the K - 1 inputs before a request's first token of this step come from its row of ``state`` ([slots, >= (K - 1) C]
+        fp32, oldest input first), which then receives the step's last K - 1 inputs. ``activation``: ``silu`` or None."""
+        self.settle()
+        self._whole(x)
+        T, C = out.shape
+        K = taps.shape[1]
+        if taps.dtype != torch.float32 or not taps.is_contiguous() or taps.shape[0] != C or x.shape[0] != T or x.shape[1] != C \
+                or out.dtype != torch.float32 or state.dtype != torch.float32 or state.stride(1) != 1 or state.shape[1] < (K - 1) * C \
+                or (bias is not None and (bias.dtype != torch.float32 or bias.numel() != C or not bias.is_contiguous())):
+            fail(EINVAL, "causal_conv: taps [channels, taps] and bias fp32, fp32 output and state, one width for all")
+        if activation not in (None, "silu"):
+            fail(ENOTSUP, f"causal_conv: activation '{activation}' is neither silu nor None")
+        self._check(self.lib.hfa_causal_conv(
+            x.data_ptr(), _code(x), _rows(x, "conv in"), taps.data_ptr(), None if bias is None else bias.data_ptr(), C, K,
+            state.data_ptr(), state.stride(0), _ints(step.q_start, "q_start", step.n_seqs + 1),
+            _ints(step.seq_slot, "seq_slot", step.n_seqs), step.n_seqs, step.max_q_len, out.data_ptr(), _rows(out, "conv out"),
+            self.ACTIVATIONS["silu"] if activation else 0, self._stream()))
+
+    def linear_scan(self, q, k, v, qk_heads, qk_dim, n_heads, v_dim, state, step, y, decay=None, step_size=None,
+                    step_bias=None, a_log=None, skip=None):
+        """The recurrence over a matrix state per head, along each request's tokens from its row of ``state`` ([slots, >=
+        heads * qk_dim * v_dim] fp32, left there for the next step): ``S <- a_t S + k_t (b_t v_t)^T``, ``y_t = S^T q_t +
+        skip[h] v_t`` (fp32). Head h reads queries and keys of head ``h // (n_heads / qk_heads)``. With ``decay`` (fp32, one
+        per head): ``a_t = decay[h]``, ``b_t = 1``. With ``step_size`` ([T, heads]), ``step_bias`` and ``a_log`` (fp32 per head):
+        ``dt = softplus(step_size + step_bias)``, ``a_t = exp(-exp(a_log) dt)``, ``b_t = dt``."""
+        self.settle()
+        for t in (q, k, v):
+            self._whole(t)
+        T = y.shape[0]
+        gate = 0 if decay is not None else 1
+        if q.dtype != k.dtype or q.dtype != v.dtype or y.dtype != torch.float32 or state.dtype != torch.float32 \
+                or state.stride(1) != 1 or q.shape[0] != T or k.shape[0] != T or v.shape[0] != T or y.shape[1] != n_heads * v_dim:
+            fail(EINVAL, "linear_scan: q, k and v of one dtype and the step's rows, fp32 output and state")
+        for t, what in ((decay, "decay"), (step_bias, "step_bias"), (a_log, "a_log"), (skip, "skip")):
+            if t is not None and (t.dtype != torch.float32 or t.numel() != n_heads or not t.is_contiguous()):
+                fail(EINVAL, f"linear_scan: {what} must be one fp32 value a head")
+        if gate == 1 and (step_size is None or step_bias is None or a_log is None or step_size.shape[0] != T):
+            fail(EINVAL, "linear_scan: without a fixed decay give step_size, step_bias and a_log")
+
+        def ptr(t):
+            return None if t is None else t.data_ptr()
+        self._check(self.lib.hfa_linear_scan(
+            q.data_ptr(), _rows(q, "scan q"), k.data_ptr(), _rows(k, "scan k"), qk_heads, qk_dim, v.data_ptr(), _rows(v, "scan v"),
+            n_heads, v_dim, _code(q), gate, ptr(decay), ptr(step_size), 0 if step_size is None else _code(step_size),
+            0 if step_size is None else _rows(step_size, "scan step"), ptr(step_bias), ptr(a_log), ptr(skip), state.data_ptr(),
+            state.stride(0), _ints(step.q_start, "q_start", step.n_seqs + 1), _ints(step.seq_slot, "seq_slot", step.n_seqs),
+            step.n_seqs, y.data_ptr(), _rows(y, "scan out"), self._stream()))
+
     # ---- layer norm, plain activations, soft cap -----------------------------------------------------------------
     def layernorm(self, x, weight, bias, eps, out, rows=None):
         """``out[r] = (x[rows[r]] - mean) / sqrt(var + eps) * weight + bias`` in fp32 (``bias`` None: no shift). A
@@ -645,10 +763,11 @@ class Ops:
             None if pend is None else self.workspace.data_ptr(), 0 if pend is None else pend.splits,
             None if pend is None or pend.bias is None else pend.bias.data_ptr(), x.shape[0], self._stream()))
 
-    ACTIVATIONS = {"gelu_erf": 1, "gelu_tanh": 2, "relu2": 3}
+    ACTIVATIONS = {"gelu_erf": 1, "gelu_tanh": 2, "relu2": 3, "silu": 4, "sigmoid": 5}
 
     def activation(self, kind, src, out):
-        """``out = act(src)`` elementwise, computed in fp32: ``gelu_erf``, ``gelu_tanh`` or ``relu2`` (relu squared)."""
+        """``out = act(src)`` elementwise, computed in fp32: ``gelu_erf``, ``gelu_tanh``, ``relu2`` (relu squared), ``silu``
+        or ``sigmoid``."""
         if kind not in self.ACTIVATIONS:
             fail(ENOTSUP, f"activation '{kind}' is not one of {', '.join(sorted(self.ACTIVATIONS))}")
         self.settle()
@@ -681,27 +800,37 @@ class Ops:
                                            ids.data_ptr(), wts.data_ptr(), self._stream()))
         return ids, wts
 
-    def moe_experts(self, h, ids, weights, w_up, w_down, act, x):
+    def moe_experts(self, h, ids, weights, w_up, w_down, act, x, gated=None):
         """``x[t] += sum_k weights[t, k] * w_down[ids[t, k]] act(w_up[ids[t, k]] h[t])``: ``w_up`` is [E, F, width],
         ``w_down`` [E, width, F]. The pairs are put in expert order on the device, each expert's rows go through the
-        two products in tiles, and the weighted results are added to ``x`` (fp32) choice by choice."""
+        two products in tiles, and the weighted results are added to ``x`` (fp32) choice by choice.
+
+        ``gated`` = (alpha, limit, shift): the experts are gated units whose weight scales their input. ``w_up`` then is
+        [E, 2F, width], an expert's gate rows before its up rows, and with ``c = weights[t, k]``, ``g = min(c Wgate h,
+        limit)``, ``u = clamp(c Wup h, -limit, limit)`` (``limit`` <= 0: unbounded) the expert gives ``Wdown (g
+        sigmoid(alpha g) (u + shift))``, unweighted; ``act`` is ignored."""
         self.settle()
         self._whole(h)
         self._source_changes(x)
         T, W = h.shape
         E, F, _ = w_up.shape
+        if gated is not None:
+            if F % 2:
+                fail(EINVAL, "moe_experts: gated experts hold gate and up rows in one matrix of 2F rows")
+            F //= 2
+        F_up = w_up.shape[1]
         top = ids.shape[1]
         n_pairs = T * top
-        if act not in self.ACTIVATIONS:
+        if gated is None and act not in self.ACTIVATIONS:
             fail(ENOTSUP, f"activation '{act}' is not one of {', '.join(sorted(self.ACTIVATIONS))}")
-        if tuple(w_up.shape) != (E, F, W) or tuple(w_down.shape) != (E, W, F) or not w_up.is_contiguous() or not w_down.is_contiguous() \
+        if tuple(w_up.shape) != (E, F_up, W) or tuple(w_down.shape) != (E, W, F) or not w_up.is_contiguous() or not w_down.is_contiguous() \
                 or w_up.dtype != w_down.dtype or (w_up.dtype != h.dtype and w_up.dtype != torch.float32) or x.dtype != torch.float32 or tuple(x.shape) != (T, W) \
                 or not x.is_contiguous() or tuple(weights.shape) != (T, top) or weights.dtype != torch.float32:
             fail(EINVAL, "moe_experts: the experts' matrices, the activations and the residual stream do not fit")
         code, wcode = _code(h), _code(w_up)              # matrices stored in 32-bit stay so beside bf16 activations
         plain = 1 if self.force_plain_gemm else 0
         # one size of tile for both products: rows are put into tiles once
-        tile_rows = 32 if plain else min(int(self.lib.hfa_moe_tile_rows(code, wcode, n_pairs, E, F, W)),
+        tile_rows = 32 if plain else min(int(self.lib.hfa_moe_tile_rows(code, wcode, n_pairs, E, F_up, W)),
                                          int(self.lib.hfa_moe_tile_rows(code, wcode, n_pairs, E, W, F)))
         max_tiles = n_pairs // tile_rows + E
         row_pair = self.scratch("moe_row_pair", (n_pairs,), torch.int32)
@@ -711,6 +840,19 @@ class Ops:
                                           n_tiles.data_ptr(), self._stream()))
         mid = self.scratch("moe_act", (n_pairs, F), h.dtype)
         y = self.scratch("moe_out", (n_pairs, W), torch.float32)
+        if gated is not None:
+            alpha, limit, shift = gated
+            sums = self.scratch("moe_gate_up", (n_pairs, F_up), torch.float32)      # 32-bit sums: the weight scales them exactly
+            self._check(self.lib.hfa_moe_gemm(h.data_ptr(), _rows(h, "moe h"), code, top, w_up.data_ptr(), wcode, row_pair.data_ptr(),
+                                              tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, sums.data_ptr(), F_up, F32, 0,
+                                              None, 0, F_up, W, plain, self._stream()))
+            self._check(self.lib.hfa_moe_gated_act(sums.data_ptr(), F_up, row_pair.data_ptr(), weights.data_ptr(), mid.data_ptr(), code, F,
+                                                   n_pairs, F, float(alpha), float(limit), float(shift), self._stream()))
+            self._check(self.lib.hfa_moe_gemm(mid.data_ptr(), F, code, 0, w_down.data_ptr(), wcode, row_pair.data_ptr(), tiles.data_ptr(),
+                                              n_tiles.data_ptr(), max_tiles, tile_rows, y.data_ptr(), W, F32, 1, None, 0, W, F,
+                                              plain, self._stream()))
+            self._check(self.lib.hfa_moe_combine(y.data_ptr(), x.data_ptr(), T, top, W, self._stream()))
+            return
         self._check(self.lib.hfa_moe_gemm(h.data_ptr(), _rows(h, "moe h"), code, top, w_up.data_ptr(), wcode, row_pair.data_ptr(),
                                           tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, mid.data_ptr(), F, code, 0, None,
                                           self.ACTIVATIONS[act], F, W, plain, self._stream()))

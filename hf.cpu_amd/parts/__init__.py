@@ -1,5 +1,5 @@
 """The parts layers are put together from. Importing this package registers them."""
 from .base import FixedState, PagedKV, ParamSpec, Part
-from . import norm, position, attention, mlp, moe, block, embedding   # noqa: F401  (registration)
+from . import norm, position, attention, recurrent, mlp, moe, block, embedding   # noqa: F401  (registration)
 
 __all__ = ["FixedState", "PagedKV", "ParamSpec", "Part"]

@@ -30,13 +30,21 @@ class Attention(Part):
     A position encoding that enters the scores instead of the queries and keys has an
     attribute ``score_slopes`` (fp32 on the device, one per query head): the score then is
     ``dot(q, k) * scale + score_slopes[h] * (pk - pq)``.
+
+    ``qk_norm`` = eps: queries and keys are RMS-normed over the whole projection (all heads at once) with the weights
+    ``q_norm`` and ``k_norm`` (names in ``names``), before the rotation. ``sink``: the softmax has one more term of score 0
+    that has no value, ``p_j = exp(s_j) / (1 + sum exp(s_i))``. ``v_mix``: ``"first"``: this layer's values, as projected,
+    are kept for the step; ``"blend"``: ``v <- (1 - l) v + l v_first`` with the scalar tensor ``v_mix`` (name in
+    ``names``) and the kept values of the same token; the blended values are what is cached. A ``"first"`` layer holds the
+    scalar too, unused.
     """
     graph_safe = True
     lazy_input_ok = True
 
 
     def __init__(self, hidden_size, n_heads, n_kv_heads, head_dim, qkv_bias, window, position,
-                 scale=None, out_bias=False, v_head_dim=None, prefix="", mask_chunk=0, own_kv=True, names=None):
+                 scale=None, out_bias=False, v_head_dim=None, prefix="", mask_chunk=0, own_kv=True, names=None,
+                 qk_norm=None, sink=False, v_mix=None):
         """``v_head_dim``: the size of a value head where it is not ``head_dim`` (key rows of the cache are
         then ``n_kv_heads * head_dim`` wide, value rows ``n_kv_heads * v_head_dim``, and the output
         projection reads ``n_heads * v_head_dim`` columns; such a mixer runs the plain kernels)."""
@@ -54,7 +62,14 @@ class Attention(Part):
         self.own_kv = bool(own_kv)
         self.names = {n: f"{n}_proj.weight" for n in "qkvo"}
         self.names.update({f"{n}_bias": f"{n}_proj.bias" for n in "qkvo"})
+        self.names.update(q_norm="q_norm.weight", k_norm="k_norm.weight", v_mix="v_mix")
         self.names.update(names or {})
+        self.qk_norm = None if qk_norm is None else float(qk_norm)
+        self.sink = bool(sink)
+        if v_mix not in (None, "first", "blend") or (v_mix and not own_kv):
+            fail(EINVAL, f"attention: v_mix '{v_mix}' is neither first nor blend, or the layer has no values of its own")
+        self.v_mix = v_mix
+        self.q_norm_w = self.k_norm_w = self.v_blend = None
         if self.window < 0 or self.mask_chunk < 0:
             fail(EINVAL, "attention: a window and a masking chunk are counted in tokens, 0 for none")
         self.scale = float(scale) if scale is not None else 1.0 / math.sqrt(head_dim)   # src/model.c:507
@@ -73,6 +88,12 @@ class Attention(Part):
             specs += [ParamSpec(p + nm[n + "_bias"], (widths[n],), "vector") for n in self._projections()]
         if self.out_bias:
             specs.append(ParamSpec(p + nm["o_bias"], (self.E,), "vector"))
+        if self.qk_norm is not None:
+            specs.append(ParamSpec(p + nm["q_norm"], (self.QD,), "vector", ("one_plus_normal", 0.1)))
+            if self.own_kv:
+                specs.append(ParamSpec(p + nm["k_norm"], (self.KD,), "vector", ("one_plus_normal", 0.1)))
+        if self.v_mix:
+            specs.append(ParamSpec(p + nm["v_mix"], (), "vector", ("normal", 0.3), optional=self.v_mix == "first"))
         return specs
 
     def _projections(self):
@@ -101,6 +122,11 @@ class Attention(Part):
         self.short_request_rows = ops.prompt_rows     # where the attention kernels for decoded tokens and for prompt portions part
         if self.out_bias:
             self.b_o = params[p + nm["o_bias"]]
+        if self.qk_norm is not None:
+            self.q_norm_w = params[p + nm["q_norm"]]
+            self.k_norm_w = params[p + nm["k_norm"]] if self.own_kv else None
+        if self.v_mix == "blend":
+            self.v_blend = params[p + nm["v_mix"]].reshape(1)
 
     def forward(self, ops, step, h, cache, x, write_cache=True):
         T = h.shape[0]
@@ -111,7 +137,17 @@ class Attention(Part):
         # a product that split K is added up inside the next kernel (position.store, the next norm)
         with ops.section("qkv"):
             ops.gemm(h, self.w_qkv[:width], qkv, bias=None if self.b_qkv is None else self.b_qkv[:width], defer=True)
-        if self.Dv == self.D:
+        prepare = {}
+        if self.qk_norm is not None:
+            prepare.update(q_norm=self.q_norm_w, k_norm=self.k_norm_w if write_cache else None, eps=self.qk_norm)
+        if self.v_mix and write_cache:
+            # the first mixing layer's values of this step's tokens wait in a work buffer for the layers that blend
+            kept = ops.scratch("v_first", (T, self.VD), ops.act_dtype)
+            prepare.update(dict(v_keep=kept) if self.v_mix == "first" else dict(v_blend=self.v_blend, v_other=kept))
+        if prepare:
+            self.position.store(ops, step, qkv, self.H, self.G if write_cache else 0, cache, write_cache, v_head_dim=self.Dv,
+                                prepare=prepare)
+        elif self.Dv == self.D:
             self.position.store(ops, step, qkv, self.H, self.G if write_cache else 0, cache, write_cache)
         else:                                   # only a position part that knows of value heads of another size can serve
             self.position.store(ops, step, qkv, self.H, self.G if write_cache else 0, cache, write_cache, v_head_dim=self.Dv)
@@ -119,6 +155,6 @@ class Attention(Part):
         with ops.section("attn"):
             ops.paged_attention(qkv, self.H, self.G, self.D, cache, step, self.window, self.scale, att,
                                 slopes=getattr(self.position, "score_slopes", None), v_head_dim=self.Dv,
-                                mask_chunk=self.mask_chunk)
+                                mask_chunk=self.mask_chunk, sink=self.sink)
         with ops.section("wo"):
             ops.gemm(att, self.w_o, x, bias=self.b_o, accumulate=True, defer=True)

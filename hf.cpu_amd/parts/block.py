@@ -20,6 +20,8 @@ class PreNormBlock(Part):
         norm_for(ops, parts["norm1"], parts["mixer"], x, h)      # also adds up a product the previous part deferred into x
         ops.settle(x)                          # (nothing left to do unless the norm could not)
         parts["mixer"].forward(ops, step, h, caches.get("mixer"), x, write_cache)
+        if "feed_forward" not in parts:         # a layer may be its mixer alone
+            return
         norm_for(ops, parts["norm2"], parts["feed_forward"], x, h)
         ops.settle(x)
         parts["feed_forward"].forward(ops, step, h, x)

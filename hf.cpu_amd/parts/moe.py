@@ -19,12 +19,22 @@ class MixtureOfExperts(Part):
 
     The experts' matrices are held stacked, [experts, ff, width] and [experts, width, ff]: one launch walks all of
     them (``Ops.moe_experts``). ``names``: the tensors' names after ``prefix`` (keys router, up, down; up and down are
-    patterns with ``{e}`` for the expert's number)."""
+    patterns with ``{e}`` for the expert's number).
+
+    ``gated`` = dict(alpha, limit, shift): the experts are gated units, ``Wdown (g sigmoid(alpha g) (u + shift))`` with
+    ``g = min(Wgate h', limit)``, ``u = clamp(Wup h', -limit, limit)`` (``limit`` <= 0: unbounded), and ``h' = weight_e h``:
+    the weight scales the expert's input, not its output (``weight_on="input"``). The gate matrices are named by
+    ``names["gate"]``; gate and up of an expert are held as one matrix, gate rows first."""
     graph_safe = True
 
     def __init__(self, hidden_size, expert_size, n_experts, top, n_groups=1, keep_groups=1, activation="relu2",
-                 scoring="softmax", renormalize=True, weight_scale=1.0, prefix="", names=None):
+                 scoring="softmax", renormalize=True, weight_scale=1.0, prefix="", names=None, gated=None,
+                 weight_on="output"):
         super().__init__(prefix)
+        if weight_on not in ("output", "input") or (weight_on == "input") != (gated is not None):
+            fail(ENOTSUP, "moe: gated experts weigh their input, experts without a gate their output; other pairings are not implemented")
+        self.gated = None if gated is None else (float(gated["alpha"]), float(gated.get("limit", 0.0)), float(gated.get("shift", 0.0)))
+        self.weight_on = weight_on
         if activation not in ("gelu_erf", "gelu_tanh", "relu2"):
             fail(ENOTSUP, f"moe: activation '{activation}' is not implemented")
         if scoring not in ("softmax", "sigmoid"):
@@ -37,7 +47,8 @@ class MixtureOfExperts(Part):
         self.n_groups, self.keep_groups = n_groups, keep_groups
         self.activation, self.scoring = activation, scoring
         self.renormalize, self.weight_scale = bool(renormalize), float(weight_scale)
-        self.names = {"router": "router.weight", "up": "experts.{e}.up_proj.weight", "down": "experts.{e}.down_proj.weight"}
+        self.names = {"router": "router.weight", "up": "experts.{e}.up_proj.weight", "down": "experts.{e}.down_proj.weight",
+                      "gate": "experts.{e}.gate_proj.weight"}
         self.names.update(names or {})
         self.w_router = self.w_up = self.w_down = None
 
@@ -48,11 +59,15 @@ class MixtureOfExperts(Part):
         specs = [ParamSpec(self._name("router"), (self.n_experts, self.E))]
         for e in range(self.n_experts):
             specs += [ParamSpec(self._name("up", e), (self.F, self.E)), ParamSpec(self._name("down", e), (self.E, self.F))]
+            if self.gated is not None:
+                specs.append(ParamSpec(self._name("gate", e), (self.F, self.E)))
         return specs
 
     def bind(self, params, ops):
         self.w_router = params[self._name("router")]
         ups = [params.pop(self._name("up", e)) for e in range(self.n_experts)]
+        if self.gated is not None:                  # an expert's gate rows, then its up rows: one product gives both
+            ups = [torch.cat([params.pop(self._name("gate", e)), u], 0) for e, u in enumerate(ups)]
         downs = [params.pop(self._name("down", e)) for e in range(self.n_experts)]
         dt = torch.float32 if any(m.dtype == torch.float32 for m in ups + downs) else ups[0].dtype
         self.w_up = memory.cat([m.to(dt).unsqueeze(0) for m in ups], 0, f"{self.prefix}up matrices of all experts")
@@ -67,4 +82,4 @@ class MixtureOfExperts(Part):
             ids, weights = ops.moe_route(logits, self.top, self.n_groups, self.keep_groups, self.scoring, self.renormalize,
                                          self.weight_scale)
         with ops.section("experts"):
-            ops.moe_experts(h, ids, weights, self.w_up, self.w_down, self.activation, x)
+            ops.moe_experts(h, ids, weights, self.w_up, self.w_down, self.activation, x, gated=self.gated)

@@ -1,5 +1,7 @@
-"""Norms of the residual stream: root mean square with a learned scale, and layer norm with scale and shift."""
+"""Norms of the residual stream: root mean square with a learned scale (whole, or in groups), and layer norm with scale
+and shift."""
 from ..registry import register_part
+from ..status import EINVAL, fail
 from .base import ParamSpec, Part
 
 
@@ -55,3 +57,28 @@ class LayerNorm(Part):
 
     def forward(self, ops, x, out, rows=None):
         ops.layernorm(x, self.weight, self.bias, self.eps, out, rows)
+
+
+@register_part("norm", "group_rmsnorm")
+class GroupRMSNorm(Part):
+    """The vector is cut into ``groups`` equal consecutive runs; each is divided by ``sqrt(mean(run^2) + eps)`` of its
+    own, and the whole is multiplied by the weight. Sums in fp32. ``weight`` is the suffix of the tensor's name after
+    ``prefix``. One group is the plain RMS norm (as a kernel of its own: nothing is left to the products around it)."""
+    graph_safe = True
+
+    def __init__(self, size, eps, groups=1, weight="weight", prefix=""):
+        super().__init__(prefix)
+        if groups <= 0 or size % groups:
+            fail(EINVAL, f"group_rmsnorm: {size} values do not form {groups} equal runs")
+        self.size, self.eps, self.groups = size, float(eps), int(groups)
+        self.weight_name = prefix + weight
+        self.weight = None
+
+    def param_specs(self):
+        return [ParamSpec(self.weight_name, (self.size,), "vector", ("one_plus_normal", 0.1))]
+
+    def bind(self, params, ops):
+        self.weight = params[self.weight_name]
+
+    def forward(self, ops, x, out, rows=None):
+        ops.group_rmsnorm(x, self.weight, self.eps, self.groups, out, rows)

@@ -11,19 +11,20 @@ from .base import Part
 
 @register_part("position", "rotary")
 class Rotary(Part):
-    """Rotation of pairs ``(i, i + rot_dim/2)`` of each head by the angle
+    """``pairing`` ``split_half``: rotation of pairs ``(i, i + rot_dim/2)`` of each head by the angle
     ``pos * theta^(-2i/rot_dim)`` (split-half pairing, src/model.c:468-493; the
     reference builds the angle by a running fp32 product, here it is one fp32
     product of the position and a table rounded from fp64). Dimensions from
     ``rot_dim`` on pass through. Values are not rotated; keys are stored rotated
-    (src/model.c:596-600)."""
+    (src/model.c:596-600). ``pairing`` ``interleaved``: the pairs are ``(2i, 2i + 1)``, the angles the same."""
     graph_safe = True
 
 
     def __init__(self, head_dim, rot_dim, theta, pairing="split_half", prefix=""):
         super().__init__(prefix)
-        if pairing != "split_half":
+        if pairing not in ("split_half", "interleaved"):
             fail(EINVAL, f"rotary pairing '{pairing}' is not implemented")
+        self.pairing = pairing
         if rot_dim % 2 or not 0 < rot_dim <= head_dim:
             fail(EINVAL, f"rotary rot_dim {rot_dim} must be even and within head_dim {head_dim}")
         self.head_dim = head_dim
@@ -39,10 +40,17 @@ class Rotary(Part):
         # layers with the same rotation share one table (and with it what a step derives from it once for all of them)
         self.inv_freq = ops.shared(("rotary frequencies", self.rot_dim, self.theta), table)
 
-    def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write, v_head_dim=None):
+    def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write, v_head_dim=None, prepare=None):
         """Rotates the queries (and keys) inside ``qkv`` at each token's position;
         if ``write``, puts each token's rotated key and its value into its cache row.
-        ``v_head_dim``: the size of a value head where it is not the keys'."""
+        ``v_head_dim``: the size of a value head where it is not the keys'. ``prepare``: what the mixer wants done to
+        queries, keys and values in the same pass (norms over the whole projections before the rotation, values
+        blended with another layer's: the keywords of ``Ops.qkv_prepare``)."""
+        if prepare or self.pairing != "split_half":
+            ops.qkv_prepare(qkv, step.positions, self.inv_freq, self.rot_dim, self.pairing, n_heads, n_kv_heads, self.head_dim,
+                            self.head_dim if v_head_dim is None else v_head_dim, cache,
+                            step.group(cache.group).slot_map if write else None, **(prepare or {}))
+            return
         ops.rope_store(qkv, step.positions, self.inv_freq, self.rot_dim, n_heads, n_kv_heads,
                        self.head_dim, cache, step.group(cache.group).slot_map if write else None, v_head_dim=v_head_dim)
 
@@ -57,7 +65,12 @@ class NoPosition(Part):
         super().__init__(prefix)
         self.head_dim = head_dim
 
-    def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write, v_head_dim=None):
+    def store(self, ops, step, qkv, n_heads, n_kv_heads, cache, write, v_head_dim=None, prepare=None):
+        if prepare:
+            ops.qkv_prepare(qkv, None, None, 0, "split_half", n_heads, n_kv_heads, self.head_dim,
+                            self.head_dim if v_head_dim is None else v_head_dim, cache,
+                            step.group(cache.group).slot_map if write else None, **prepare)
+            return
         if write:
             ops.rope_store(qkv, step.positions, None, 0, n_heads, n_kv_heads, self.head_dim,
                            cache, step.group(cache.group).slot_map, v_head_dim=v_head_dim)
