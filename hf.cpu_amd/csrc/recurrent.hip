@@ -60,7 +60,7 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const T* __restrict__ 
 extern "C" int hfa_causal_conv(const void* in, int dtype, int ld_in, const float* taps, const float* bias, int n_channels,
                                int n_taps, float* state, size_t state_ld, const int* q_start, const int* seq_slot, int n_seqs,
                                int max_q_len, float* out, int ldo, int act, hipStream_t stream) {
-    HFA_REQUIRE(in && taps && state && q_start && seq_slot && out && n_channels > 0 && n_seqs > 0 && max_q_len > 0,
+    HFA_REQUIRE(in && taps && (state || n_taps == 1) && q_start && seq_slot && out && n_channels > 0 && n_seqs > 0 && max_q_len > 0,
                 "causal_conv: bad arguments");
     HFA_REQUIRE(n_taps >= 1 && n_taps <= CONV_MAX_TAPS, "causal_conv: %d taps (1 to %d)", n_taps, CONV_MAX_TAPS);
     HFA_REQUIRE(ld_in >= n_channels && ldo >= n_channels && state_ld >= (size_t)(n_taps - 1) * n_channels,

@@ -79,6 +79,7 @@ def write_safetensors(path, tensors, dtype="F32"):
     """The tests' own writer (8-byte length, JSON header, raw data)."""
     header, blobs, off = {}, [], 0
     for name, a in tensors.items():
+        shape = list(np.shape(a))                       # (a scalar keeps its empty shape)
         a = np.ascontiguousarray(a, dtype=np.float32)
         if dtype == "BF16":
             raw = (bf16_round(a).view(np.uint32) >> 16).astype("<u2").tobytes()
@@ -86,7 +87,7 @@ def write_safetensors(path, tensors, dtype="F32"):
             raw = a.astype("<f2").tobytes()
         else:
             raw = a.astype("<f4").tobytes()
-        header[name] = {"dtype": dtype, "shape": list(a.shape), "data_offsets": [off, off + len(raw)]}
+        header[name] = {"dtype": dtype, "shape": shape, "data_offsets": [off, off + len(raw)]}
         off += len(raw)
         blobs.append(raw)
     h = json.dumps(header).encode()
