@@ -1,7 +1,7 @@
-"""``bench.py --design goridra``: prefill and decode of the Goridra design at sizes that resemble a real model's layers
-(random weights), beside Qwen2 dense at equal width, heads and layer count, with every part of a step priced against
-its roofline: flops / time against the matrix cores for a prefill's parts, bytes / time against HBM for a decode
-step's. One JSON line a size."""
+"""``bench.py --design goridra | tobozen``: prefill and decode of a design at sizes that resemble a real model's layers
+(random weights), beside the closest other design at equal width, heads and layer count (Goridra beside Qwen2 dense,
+Tobozen beside Goridra), with every part of a step priced against its roofline: flops / time against the matrix cores
+for a prefill's parts, bytes / time against HBM for a decode step's. One JSON line a size."""
 import json
 import math
 import sys
@@ -12,12 +12,54 @@ MFMA_PEAK = 2.5e15
 PROMPT, PAGE = 2048, 16
 
 # width, heads, key/value heads, head size, dense ff, experts, choices, groups, kept groups, expert ff, layers, vocabulary
+# (for Tobozen also: heads, head size, state and groups of the state-space layers; layers come in threes)
 SIZES = {
     "2k": dict(width=2048, heads=16, kv_heads=4, dim=128, ff=8192, experts=32, top=4, groups=4, keep=2, expert_ff=1024,
-               layers=8, vocab=32000, mask=1024),
+               layers=8, vocab=32000, mask=1024, ssm_heads=64, ssm_dim=64, ssm_state=128, ssm_groups=8, triples=2),
     "4k": dict(width=4096, heads=32, kv_heads=8, dim=128, ff=14336, experts=64, top=8, groups=8, keep=4, expert_ff=1024,
-               layers=4, vocab=32000, mask=1024),
+               layers=4, vocab=32000, mask=1024, ssm_heads=128, ssm_dim=64, ssm_state=128, ssm_groups=8, triples=1),
 }
+
+
+def tobozen_shape(z):
+    """Layers in threes: a state-space layer (inner width twice the model's), softmax attention, linear attention; each
+    with a mixture of experts."""
+    H, G, D = z["heads"], z["kv_heads"], z["dim"]
+    moe = dict(kind="moe", expert=dict(ff=z["expert_ff"], limit=7.0), router=dict(experts=z["experts"], top=z["top"]))
+    three = [
+        dict(type="mamba2", mixer=dict(heads=z["ssm_heads"], vdim=z["ssm_dim"], state=z["ssm_state"], groups=z["ssm_groups"], conv=4,
+                                       norm_groups=z["ssm_groups"]), mlp=moe),
+        dict(type="attention", mixer=dict(heads=H, kv_heads=G, dim=D, vdim=D, scale=1.0 / math.sqrt(D), rot=dict(dims=D, base=500000.0),
+                                          v_mix=True), mlp=moe),
+        dict(type="lightning", mixer=dict(heads=H, dim=D, vdim=D, decay=[1.0 - 2.0 ** -(3 + 8 * h // H) for h in range(H)]), mlp=moe)]
+    return dict(architecture="Tobozen", vocab=z["vocab"], width=z["width"], norm=dict(eps=1e-6, groups=2), layers=three * z["triples"])
+
+
+def tobozen_work(z, T, batch, ctx):
+    """({part: flops of a prefill of T tokens}, {part: bytes of a decode step}), all layers together, bf16. The
+    recurrences are priced by the products of their state updates and outputs (4 N P a head and token) in a prefill and
+    by their fp32 states, read and written once a request, in a decode step."""
+    W, H, G, D, V, n3 = z["width"], z["heads"], z["kv_heads"], z["dim"], z["vocab"], z["triples"]
+    QD, KD = H * D, G * D
+    SH, SP, SN, SG = z["ssm_heads"], z["ssm_dim"], z["ssm_state"], z["ssm_groups"]
+    inner = SH * SP
+    w_in = 2 * inner + 2 * SG * SN + SH
+    E, top, F = z["experts"], z["top"], z["expert_ff"]
+    L = 3 * n3
+    params = {"qkv": n3 * W * (QD + 2 * KD), "wo": n3 * QD * W, "ssm_in": n3 * W * w_in, "ssm_wo": n3 * inner * W,
+              "lin_qkv": n3 * W * 4 * QD, "lin_wo": n3 * QD * W, "router": L * E * W, "head": V * W}
+    pre = {k: 2.0 * T * v for k, v in params.items() if k != "head"}
+    pre["attn"] = n3 * 4.0 * D * H * T * (T + 1) / 2
+    pre["ssm_scan"] = n3 * T * SH * 4.0 * SN * SP
+    pre["lin_scan"] = n3 * T * H * 4.0 * D * D
+    pre["experts"] = L * T * top * 6.0 * F * W
+    dec = {k: 2.0 * v for k, v in params.items()}
+    touched = E * (1.0 - (1.0 - top / E) ** batch)
+    dec["experts"] = L * touched * 3 * F * W * 2.0
+    dec["attn"] = batch * ctx * 2 * KD * n3 * 2.0
+    dec["ssm_scan"] = batch * n3 * SH * SN * SP * 4 * 2.0
+    dec["lin_scan"] = batch * n3 * H * D * D * 4 * 2.0
+    return pre, dec
 
 
 def goridra_shape(z):
@@ -52,6 +94,8 @@ def qwen2_shape(z):
 def part_work(design, z, T, batch, ctx):
     """({part: flops of a prefill of T tokens}, {part: bytes of a decode step of `batch` requests at context `ctx`}),
     all layers together, bf16."""
+    if design == "tobozen":
+        return tobozen_work(z, T, batch, ctx)
     W, H, G, D, L, V = z["width"], z["heads"], z["kv_heads"], z["dim"], z["layers"], z["vocab"]
     QD, KD = H * D, G * D
     if design == "qwen2":
@@ -88,7 +132,11 @@ def run(args):
     for size in (args.sizes.split(",") if args.sizes else list(SIZES)):
         z = SIZES[size]
         line = {"size": size, "dims": z, "context": context, "dtype": "bf16", "data": "synthetic"}
-        for design, shape in (("goridra", goridra_shape(z)), ("qwen2", qwen2_shape(z))):
+        shapes = {"goridra": goridra_shape, "qwen2": qwen2_shape, "tobozen": tobozen_shape}
+        beside = {"goridra": "qwen2", "tobozen": "goridra"}[args.design]
+        if args.design == "tobozen":                 # the same number of layers in both designs
+            z = dict(z, layers=3 * z["triples"])
+        for design, shape in ((args.design, shapes[args.design](z)), (beside, shapes[beside](z))):
             cfg = hf_cpu_amd.config_from_dict(shape)
             batches = [int(b) for b in args.batches.split(",")]
             s = S.Session(cfg, dtype="bfloat16", ctx_max=context + 64, batch=PROMPT, page_size=PAGE, max_seqs=max(batches),

@@ -148,12 +148,14 @@ int hfa_qkv_prepare(void* qkv, int dtype, int ld, const int* positions, const fl
 // hfa_causal_conv: out[t, c] = act(bias[c] + sum_j taps[c, j] in[t - (K - 1) + j, c]) (fp32 out; act HFA_ACT_SILU or none);
 // inputs before the step's first token come from the state row ([K - 1][C], oldest first), which then receives the
 // step's last K - 1 inputs.
-// hfa_linear_scan: per head h (keys and queries of head h / (n_heads / qk_heads)), S [qk_dim][v_dim] in the state row:
+// hfa_linear_scan: per head h (keys and queries of head h / (n_heads / qk_heads)), S [qk_dim][v_dim] in the state row (in the
+// kernel's own order, padded: hfa_linear_scan_state_floats values a row, zero for a new request; qk_dim at most 256):
 // S <- a_t S + k_t (b_t v_t)^T, y_t = S^T q_t + skip[h] v_t (skip null: 0). gate 0: a_t = decay[h], b_t = 1. gate 1:
 // dt = softplus(step[t, h] + step_bias[h]), a_t = exp(-exp(a_log[h]) dt), b_t = dt. y fp32.
 int hfa_causal_conv(const void* in, int dtype, int ld_in, const float* taps, const float* bias, int n_channels, int n_taps,
                     float* state, size_t state_ld, const int* q_start, const int* seq_slot, int n_seqs, int max_q_len, float* out,
                     int ldo, int act, hipStream_t stream);
+size_t hfa_linear_scan_state_floats(int n_heads, int qk_dim, int v_dim);
 int hfa_linear_scan(const void* q, int ldq, const void* k, int ldk, int qk_heads, int qk_dim, const void* v, int ldv, int n_heads,
                     int v_dim, int dtype, int gate, const float* decay, const void* step, int step_dtype, int ld_step,
                     const float* step_bias, const float* a_log, const float* skip, float* state, size_t state_ld,

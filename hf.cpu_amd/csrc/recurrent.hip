@@ -80,58 +80,103 @@ extern "C" int hfa_causal_conv(const void* in, int dtype, int ld_in, const float
 }
 
 // ---- the linear recurrence ------------------------------------------------------------------------------------
-// One block a (request, head). The state S [N][P] of the head lives in registers for the whole walk: thread (p, ns)
-// holds S[n][p] for the n of its slice (n = ns, ns + 4, ...: the four slices of a column sit in neighbouring lanes, and
-// a token's output is their sum). The tokens' k, q, v, a and b are staged through LDS SCAN_TOKENS at a time.
+// A block of four waves owns 256 / NS columns p of one head's state S [N][P] of one request and walks the request's
+// tokens in order. A column is spread over NS neighbouring lanes: lane ns holds S[n][p] for the NPT values n = ns NPT
+// + i in registers for the whole walk, and a token's output is the sum over the NS lanes. The tokens' k, q, v, a and b
+// are staged through LDS SCAN_TOKENS at a time; the next tokens' loads are on their way while these are walked. Inside
+// the walk nothing crosses lanes: every lane leaves its share of a token's output in LDS, and after SCAN_TOKENS tokens
+// the shares are added up (lane 0's first, in a fixed order) and the outputs leave as whole runs of columns, so the
+// only chain from token to token is the one the recurrence itself has.
+//
+// In the state row a head's values lie in the order the lanes read them: value (n = ns NPT + i, p) of head h at
+// (h NPT + i) * P_pad * NS + p * NS + ns, with P_pad = P rounded up to whole blocks and n padded to NS NPT (the
+// padding stays zero): a wave reads and writes whole lines. NS and NPT follow from N alone (scan_shape), so every
+// step finds the layout that the step before left; hfa_linear_scan_state_floats gives the size of a row.
 //
 // gate 0: a_t = decay[h], b_t = 1 (a fixed decay per head).
 // gate 1: dt = softplus(step[t, h] + step_bias[h]), a_t = exp(-exp(a_log[h]) dt), b_t = dt (a step size per token).
-#define SCAN_NS 4
 #define SCAN_TOKENS 16
-template <typename T, typename TS, int NPT>
-__global__ __launch_bounds__(1024) void linear_scan_kernel(
+#define SCAN_THREADS 256
+
+// Up to sixteen lanes a column with 4, 8 or 16 values each. (Four values a lane on up to 64 lanes a column, which puts
+// four times the waves on a SIMD for states of 128 rows, was measured: a prompt of 2,048 tokens 17 % quicker at 64 heads,
+// 50 % slower at 128 heads, decode steps of 64 requests 50 % slower: more blocks, each with the same staging and barriers.)
+static void scan_shape(int N, int* ns, int* npt) {
+    *ns = N >= 64 ? 16 : N > 16 ? 8 : 4;
+    const int per = (N + *ns - 1) / *ns;
+    *npt = per <= 4 ? 4 : per <= 8 ? 8 : 16;
+}
+
+extern "C" size_t hfa_linear_scan_state_floats(int n_heads, int qk_dim, int v_dim) {
+    int ns, npt;
+    scan_shape(qk_dim, &ns, &npt);
+    const int pt = SCAN_THREADS / ns, p_pad = (v_dim + pt - 1) / pt * pt;
+    return (size_t)n_heads * ns * npt * p_pad;
+}
+
+template <typename T, typename TS, int NS, int NPT>
+__global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(
     const T* __restrict__ q, int ldq, const T* __restrict__ k, int ldk, int heads_per_qk, int N, const T* __restrict__ v,
     int ldv, int P, int gate, const float* __restrict__ decay, const TS* __restrict__ step, int ld_step,
     const float* __restrict__ step_bias, const float* __restrict__ a_log, const float* __restrict__ skip,
     float* __restrict__ state, size_t state_ld, const int* __restrict__ q_start, const int* __restrict__ seq_slot,
     float* __restrict__ y, int ldy) {
-    extern __shared__ float lds[];
-    const int h = blockIdx.x, s = blockIdx.y, tid = threadIdx.x;
-    const int p = tid / SCAN_NS, ns = tid % SCAN_NS;
+    constexpr int NPAD = NS * NPT, PT = SCAN_THREADS / NS, TOK = SCAN_TOKENS;
+    constexpr int RK = TOK * NPAD / SCAN_THREADS, RV = (TOK * PT + SCAN_THREADS - 1) / SCAN_THREADS;
+    static_assert(TOK * NPAD % SCAN_THREADS == 0 && NPT % 4 == 0, "the staging loops are whole");
+    __shared__ __attribute__((aligned(16))) float k_s[TOK * NPAD];
+    __shared__ __attribute__((aligned(16))) float q_s[TOK * NPAD];
+    __shared__ float v_s[TOK * PT];
+    __shared__ float a_s[TOK], b_s[TOK];
+    __shared__ __attribute__((aligned(16))) float part_s[TOK * SCAN_THREADS];      // [token][column][lane of the column]
+    const int h = blockIdx.x, s = blockIdx.y, pz = blockIdx.z, tid = threadIdx.x;
+    const int pl = tid / NS, ns = tid % NS;
     const int q0 = q_start[s], n_tok = q_start[s + 1] - q0;
     if (n_tok <= 0) return;
-    float* k_s = lds;                                   // [SCAN_TOKENS][N]
-    float* q_s = k_s + SCAN_TOKENS * N;                 // [SCAN_TOKENS][N]
-    float* v_s = q_s + SCAN_TOKENS * N;                 // [SCAN_TOKENS][P]
-    float* a_s = v_s + SCAN_TOKENS * P;                 // [SCAN_TOKENS]
-    float* b_s = a_s + SCAN_TOKENS;                     // [SCAN_TOKENS]
-    const int g = h / heads_per_qk;
-    float* S = state + (size_t)seq_slot[s] * state_ld + (size_t)h * N * P;
-    const bool live = p < P;
+    const int g = h / heads_per_qk, p_pad = (int)gridDim.z * PT;
+    float* S = state + (size_t)seq_slot[s] * state_ld + (size_t)h * NPT * p_pad * NS + (size_t)pz * SCAN_THREADS + tid;
     float st[NPT];
 #pragma unroll
-    for (int i = 0; i < NPT; i++) {
-        const int n = ns + SCAN_NS * i;
-        st[i] = live && n < N ? S[(size_t)n * P + p] : 0.f;
-    }
+    for (int i = 0; i < NPT; i++) st[i] = S[(size_t)i * p_pad * NS];
     const float d = skip ? skip[h] : 0.f;
     const float head_decay = gate == 0 ? decay[h] : 0.f;
     const float neg_rate = gate == 1 ? -expf(a_log[h]) : 0.f, sb = gate == 1 ? step_bias[h] : 0.f;
-    for (int c0 = 0; c0 < n_tok; c0 += SCAN_TOKENS) {
-        const int nt = n_tok - c0 < SCAN_TOKENS ? n_tok - c0 : SCAN_TOKENS;
-        __syncthreads();
-        for (int i = tid; i < nt * N; i += blockDim.x) {
-            const int t = i / N, n = i % N;
-            k_s[i] = to_f32(k[(size_t)(q0 + c0 + t) * ldk + g * N + n]);
-            q_s[i] = to_f32(q[(size_t)(q0 + c0 + t) * ldq + g * N + n]);
+    const T* kg = k + (size_t)q0 * ldk + g * N;
+    const T* qg = q + (size_t)q0 * ldq + g * N;
+    const T* vg = v + (size_t)q0 * ldv + h * P + pz * PT;
+    // Two sets of registers take turns: while one chunk of tokens is walked, the loads of the next two are on their way
+    // (a trip to memory takes longer than the walk of one chunk).
+    struct Staged { float k[RK], q[RK], v[RV], step; };
+    Staged set_a, set_b;
+    // the tokens c0 .. c0 + TOK - 1 into registers (zeros beyond the request's tokens, beyond N and beyond P)
+    auto fetch = [&](Staged& g_, int c0) {
+        if (c0 >= n_tok) return;
+#pragma unroll
+        for (int r = 0; r < RK; r++) {
+            const int idx = tid + r * SCAN_THREADS, t = c0 + idx / NPAD, n = idx % NPAD;
+            const bool ok = t < n_tok && n < N;
+            g_.k[r] = ok ? to_f32(kg[(size_t)t * ldk + n]) : 0.f;
+            g_.q[r] = ok ? to_f32(qg[(size_t)t * ldq + n]) : 0.f;
         }
-        for (int i = tid; i < nt * P; i += blockDim.x) {
-            const int t = i / P, pp = i % P;
-            v_s[i] = to_f32(v[(size_t)(q0 + c0 + t) * ldv + h * P + pp]);
+#pragma unroll
+        for (int r = 0; r < RV; r++) {
+            const int idx = tid + r * SCAN_THREADS, t = c0 + idx / PT, pp = idx % PT;
+            g_.v[r] = (idx < TOK * PT && t < n_tok && pz * PT + pp < P) ? to_f32(vg[(size_t)t * ldv + pp]) : 0.f;
         }
-        if (tid < nt) {
+        g_.step = (gate == 1 && tid < TOK && c0 + tid < n_tok) ? to_f32(step[(size_t)(q0 + c0 + tid) * ld_step + h]) : 0.f;
+    };
+    auto stash = [&](const Staged& g_) {
+#pragma unroll
+        for (int r = 0; r < RK; r++) {
+            k_s[tid + r * SCAN_THREADS] = g_.k[r];
+            q_s[tid + r * SCAN_THREADS] = g_.q[r];
+        }
+#pragma unroll
+        for (int r = 0; r < RV; r++)
+            if (tid + r * SCAN_THREADS < TOK * PT) v_s[tid + r * SCAN_THREADS] = g_.v[r];
+        if (tid < TOK) {
             if (gate == 1) {
-                const float z = to_f32(step[(size_t)(q0 + c0 + tid) * ld_step + h]) + sb;
+                const float z = g_.step + sb;
                 const float dt = fmaxf(z, 0.f) + log1pf(expf(-fabsf(z)));          // softplus, exact for every z
                 a_s[tid] = expf(neg_rate * dt);
                 b_s[tid] = dt;
@@ -140,33 +185,61 @@ __global__ __launch_bounds__(1024) void linear_scan_kernel(
                 b_s[tid] = 1.f;
             }
         }
+    };
+    auto chunk = [&](Staged& g_, int c0) {
+        const int nt = n_tok - c0 < TOK ? n_tok - c0 : TOK;
+        __syncthreads();                                   // the walk before has read what is overwritten now
+        stash(g_);
         __syncthreads();
-        if (!live) continue;
-        for (int t = 0; t < nt; t++) {
-            const float a = a_s[t], vt = v_s[t * P + p], bv = b_s[t] * vt;
-            const float* kt = k_s + t * N;
-            const float* qt = q_s + t * N;
+        fetch(g_, c0 + 2 * TOK);
+        auto token = [&](int t) {
+            const float a = a_s[t], bv = b_s[t] * v_s[t * PT + pl];
+            const float4* kt = reinterpret_cast<const float4*>(k_s + t * NPAD + ns * NPT);
+            const float4* qt = reinterpret_cast<const float4*>(q_s + t * NPAD + ns * NPT);
+            float acc0 = 0.f, acc1 = 0.f;
+#pragma unroll
+            for (int i = 0; i < NPT / 4; i++) {
+                const float4 kk = kt[i], qq = qt[i];
+                st[4 * i] = fmaf(a, st[4 * i], kk.x * bv);
+                st[4 * i + 1] = fmaf(a, st[4 * i + 1], kk.y * bv);
+                st[4 * i + 2] = fmaf(a, st[4 * i + 2], kk.z * bv);
+                st[4 * i + 3] = fmaf(a, st[4 * i + 3], kk.w * bv);
+                acc0 = fmaf(st[4 * i], qq.x, acc0);
+                acc1 = fmaf(st[4 * i + 1], qq.y, acc1);
+                acc0 = fmaf(st[4 * i + 2], qq.z, acc0);
+                acc1 = fmaf(st[4 * i + 3], qq.w, acc1);
+            }
+            part_s[t * SCAN_THREADS + tid] = acc0 + acc1;
+        };
+        if (nt == TOK) {
+#pragma unroll 4
+            for (int t = 0; t < TOK; t++) token(t);
+        } else {
+            for (int t = 0; t < nt; t++) token(t);
+        }
+        __syncthreads();
+        // the outputs of the tokens just walked: thread -> (token, column), the lanes' shares added in lane order
+        for (int idx = tid; idx < nt * PT; idx += SCAN_THREADS) {
+            const int t = idx / PT, pp = idx % PT;
+            if (pz * PT + pp >= P) continue;
+            const float4* sh = reinterpret_cast<const float4*>(part_s + t * SCAN_THREADS + pp * NS);
             float acc = 0.f;
 #pragma unroll
-            for (int i = 0; i < NPT; i++) {
-                const int n = ns + SCAN_NS * i;
-                if (n < N) {
-                    st[i] = fmaf(a, st[i], kt[n] * bv);
-                    acc = fmaf(st[i], qt[n], acc);
-                }
+            for (int i = 0; i < NS / 4; i++) {
+                const float4 u = sh[i];
+                acc = ((acc + u.x) + u.y) + u.z + u.w;
             }
-            acc += __shfl_xor(acc, 1, WAVE);
-            acc += __shfl_xor(acc, 2, WAVE);
-            if (ns == 0) y[(size_t)(q0 + c0 + t) * ldy + h * P + p] = fmaf(d, vt, acc);
+            y[(size_t)(q0 + c0 + t) * ldy + h * P + pz * PT + pp] = fmaf(d, v_s[t * PT + pp], acc);
         }
+    };
+    fetch(set_a, 0);
+    fetch(set_b, TOK);
+    for (int c0 = 0; c0 < n_tok; c0 += 2 * TOK) {
+        chunk(set_a, c0);
+        if (c0 + TOK < n_tok) chunk(set_b, c0 + TOK);
     }
-    if (live) {
 #pragma unroll
-        for (int i = 0; i < NPT; i++) {
-            const int n = ns + SCAN_NS * i;
-            if (n < N) S[(size_t)n * P + p] = st[i];
-        }
-    }
+    for (int i = 0; i < NPT; i++) S[(size_t)i * p_pad * NS] = st[i];
 }
 
 extern "C" int hfa_linear_scan(const void* q, int ldq, const void* k, int ldk, int qk_heads, int qk_dim, const void* v,
@@ -177,30 +250,31 @@ extern "C" int hfa_linear_scan(const void* q, int ldq, const void* k, int ldk, i
     HFA_REQUIRE(q && k && v && state && q_start && seq_slot && y && n_seqs > 0, "linear_scan: a null argument");
     HFA_REQUIRE(n_heads > 0 && qk_heads > 0 && n_heads % qk_heads == 0 && qk_dim > 0 && v_dim > 0,
                 "linear_scan: %d heads over %d heads of keys", n_heads, qk_heads);
+    HFA_REQUIRE(qk_dim <= 256, "linear_scan: a state of %d rows a head is too large (at most 256)", qk_dim);
     HFA_REQUIRE(ldq >= qk_heads * qk_dim && ldk >= qk_heads * qk_dim && ldv >= n_heads * v_dim && ldy >= n_heads * v_dim &&
-                    state_ld >= (size_t)n_heads * qk_dim * v_dim, "linear_scan: a row is shorter than its heads");
-    HFA_REQUIRE(qk_dim <= SCAN_NS * 64 && v_dim <= 1024 / SCAN_NS, "linear_scan: a state of %d x %d a head is too large (at most %d x %d)",
-                qk_dim, v_dim, SCAN_NS * 64, 1024 / SCAN_NS);
+                    state_ld >= hfa_linear_scan_state_floats(n_heads, qk_dim, v_dim),
+                "linear_scan: a row is shorter than its heads (a state row holds hfa_linear_scan_state_floats values)");
     HFA_REQUIRE(dtype == HFA_F32 || dtype == HFA_BF16, "linear_scan: unknown dtype %d", dtype);
     HFA_REQUIRE((gate == 0 && decay) || (gate == 1 && step && step_bias && a_log && ld_step >= n_heads &&
                                          (step_dtype == HFA_F32 || step_dtype == HFA_BF16)),
                 "linear_scan: gate 0 needs a decay per head, gate 1 step sizes, their bias and the logarithm of the rate");
-    HFA_REQUIRE(n_heads <= 65535 && n_seqs <= 65535, "linear_scan: the step exceeds the grid");
-    const int threads = (v_dim * SCAN_NS + WAVE - 1) / WAVE * WAVE;
-    const size_t smem = (size_t)(SCAN_TOKENS * (2 * qk_dim + v_dim + 2)) * sizeof(float);
-    const int per = (qk_dim + SCAN_NS - 1) / SCAN_NS;
-    dim3 grid(n_heads, n_seqs);
-#define SCAN_GO(T, TS, NPT)                                                                                              \
-    linear_scan_kernel<T, TS, NPT><<<grid, threads, smem, stream>>>(                                                     \
+    int ns, npt;
+    scan_shape(qk_dim, &ns, &npt);
+    const int pt = SCAN_THREADS / ns, p_tiles = (v_dim + pt - 1) / pt;
+    HFA_REQUIRE(n_heads <= 65535 && n_seqs <= 65535 && p_tiles <= 65535, "linear_scan: the step exceeds the grid");
+    dim3 grid(n_heads, n_seqs, p_tiles);
+#define SCAN_GO(T, TS, NS, NPT)                                                                                          \
+    linear_scan_kernel<T, TS, NS, NPT><<<grid, SCAN_THREADS, 0, stream>>>(                                               \
         (const T*)q, ldq, (const T*)k, ldk, n_heads / qk_heads, qk_dim, (const T*)v, ldv, v_dim, gate, decay, (const TS*)step, \
         ld_step, step_bias, a_log, skip, state, state_ld, q_start, seq_slot, y, ldy)
-#define SCAN_SIZES(T, TS)                        \
-    do {                                         \
-        if (per <= 4) SCAN_GO(T, TS, 4);         \
-        else if (per <= 8) SCAN_GO(T, TS, 8);    \
-        else if (per <= 16) SCAN_GO(T, TS, 16);  \
-        else if (per <= 32) SCAN_GO(T, TS, 32);  \
-        else SCAN_GO(T, TS, 64);                 \
+#define SCAN_SIZES(T, TS)                                          \
+    do {                                                           \
+        if (ns == 4) SCAN_GO(T, TS, 4, 4);                         \
+        else if (ns == 8 && npt == 4) SCAN_GO(T, TS, 8, 4);        \
+        else if (ns == 8) SCAN_GO(T, TS, 8, 8);                    \
+        else if (npt == 4) SCAN_GO(T, TS, 16, 4);                  \
+        else if (npt == 8) SCAN_GO(T, TS, 16, 8);                  \
+        else SCAN_GO(T, TS, 16, 16);                               \
     } while (0)
     if (dtype == HFA_F32) { if (step_dtype == HFA_BF16 && gate == 1) SCAN_SIZES(float, bf16); else SCAN_SIZES(float, float); }
     else { if (step_dtype == HFA_F32 && gate == 1) SCAN_SIZES(bf16, float); else SCAN_SIZES(bf16, bf16); }

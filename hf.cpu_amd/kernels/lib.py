@@ -72,6 +72,8 @@ def library():
             lib.hfa_probe_mfma_threads.argtypes = []
             lib.hfa_attention_prompt_rows.restype = c_int
             lib.hfa_attention_prompt_rows.argtypes = []
+            lib.hfa_linear_scan_state_floats.restype = c_size_t
+            lib.hfa_linear_scan_state_floats.argtypes = [c_int] * 3
             lib.hfa_moe_tile_rows.restype = c_int
             lib.hfa_moe_tile_rows.argtypes = [c_int] * 6
             for name, args in _SIGNATURES.items():

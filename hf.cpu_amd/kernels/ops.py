@@ -711,10 +711,21 @@ class Ops:
             _ints(step.seq_slot, "seq_slot", step.n_seqs), step.n_seqs, step.max_q_len, out.data_ptr(), _rows(out, "conv out"),
             self.ACTIVATIONS["silu"] if activation else 0, self._stream()))
 
+    @staticmethod
+    def scan_state_floats(n_heads, qk_dim, v_dim):
+        """The fp32 values of a request's state row that ``linear_scan`` needs for ``n_heads`` states of ``qk_dim`` x ``v_dim``:
+        the kernel keeps them in the order its lanes read them, both sizes padded to what a block walks (the library's
+        ``hfa_linear_scan_state_floats``, mirrored here so that a cache can be planned without the library)."""
+        lanes = 16 if qk_dim >= 64 else 8 if qk_dim > 16 else 4
+        per = -(-qk_dim // lanes)
+        per = 4 if per <= 4 else 8 if per <= 8 else 16
+        columns = 256 // lanes
+        return n_heads * lanes * per * (-(-v_dim // columns) * columns)
+
     def linear_scan(self, q, k, v, qk_heads, qk_dim, n_heads, v_dim, state, step, y, decay=None, step_size=None,
                     step_bias=None, a_log=None, skip=None):
         """The recurrence over a matrix state per head, along each request's tokens from its row of ``state`` ([slots, >=
-        heads * qk_dim * v_dim] fp32, left there for the next step): ``S <- a_t S + k_t (b_t v_t)^T``, ``y_t = S^T q_t +
+        ``scan_state_floats``] fp32, in the kernel's own order, left there for the next step): ``S <- a_t S + k_t (b_t v_t)^T``, ``y_t = S^T q_t +
         skip[h] v_t`` (fp32). Head h reads queries and keys of head ``h // (n_heads / qk_heads)``. With ``decay`` (fp32, one
         per head): ``a_t = decay[h]``, ``b_t = 1``. With ``step_size`` ([T, heads]), ``step_bias`` and ``a_log`` (fp32 per head):
         ``dt = softplus(step_size + step_bias)``, ``a_t = exp(-exp(a_log) dt)``, ``b_t = dt``."""
@@ -729,6 +740,8 @@ class Ops:
         for t, what in ((decay, "decay"), (step_bias, "step_bias"), (a_log, "a_log"), (skip, "skip")):
             if t is not None and (t.dtype != torch.float32 or t.numel() != n_heads or not t.is_contiguous()):
                 fail(EINVAL, f"linear_scan: {what} must be one fp32 value a head")
+        if state.shape[1] < self.scan_state_floats(n_heads, qk_dim, v_dim) or qk_dim > 256:
+            fail(EINVAL, f"linear_scan: a state row of {state.shape[1]} values for {n_heads} states of {qk_dim} x {v_dim} (at most 256 rows)")
         if gate == 1 and (step_size is None or step_bias is None or a_log is None or step_size.shape[0] != T):
             fail(EINVAL, "linear_scan: without a fixed decay give step_size, step_bias and a_log")
 

@@ -4,6 +4,7 @@ kernel for the recurrence (``Ops.linear_scan``): ``S <- a_t S + k_t (b_t v_t)^T`
 import torch
 
 from .. import memory
+from ..kernels.ops import Ops
 from ..registry import register_part
 from ..status import EINVAL, fail
 from .base import FixedState, ParamSpec, Part
@@ -35,7 +36,7 @@ class Mamba2(Part):
         self.norm_groups, self.eps = norm_groups, float(eps)
         self.C = self.inner + 2 * n_groups * state_size            # channels of the convolution
         self.W_in = 2 * self.inner + 2 * n_groups * state_size + n_heads
-        self.n_scan = n_heads * state_size * head_dim              # floats of the recurrence in a state row; the convolution's follow
+        self.n_scan = Ops.scan_state_floats(n_heads, state_size, head_dim)    # of the recurrence in a state row; the convolution's follow
         self.names = {"in": "in_proj.weight", "conv": "conv.weight", "conv_bias": "conv.bias", "dt_bias": "dt_bias",
                       "a_log": "A_log", "d": "D", "norm": "norm.weight", "o": "out_proj.weight"}
         self.names.update(names or {})
@@ -81,7 +82,7 @@ class Mamba2(Part):
         gated = ops.scratch("ssm_gated", (T, inner), ops.act_dtype)
         with ops.section("ssm_norm"):
             ops.group_rmsnorm(y, self.norm_w, self.eps, self.norm_groups, gated, gate=proj[:, :inner], gate_kind="silu_before")
-        with ops.section("wo"):
+        with ops.section("ssm_wo"):
             ops.gemm(gated, self.w_o, x, accumulate=True, defer=True)
 
 
@@ -114,7 +115,7 @@ class LightningAttention(Part):
                 ParamSpec(p + nm["o"], (self.E, VD))]
 
     def cache_need(self):
-        return FixedState(self.H * self.D * self.Dv)
+        return FixedState(Ops.scan_state_floats(self.H, self.D, self.Dv))
 
     def bind(self, params, ops):
         p, nm = self.prefix, self.names
@@ -131,7 +132,7 @@ class LightningAttention(Part):
         T, QD, VD = h.shape[0], self.H * self.D, self.H * self.Dv
         qkv = ops.scratch("lin_qkv", (T, 2 * QD + VD), ops.act_dtype)
         gate = ops.scratch("lin_gate", (T, VD), ops.act_dtype)
-        with ops.section("qkv"):
+        with ops.section("lin_qkv"):
             ops.gemm(h, self.w_qkv, qkv, activation="silu")
             ops.gemm(h, self.w_g, gate)
         o = ops.scratch("lin_o", (T, VD), torch.float32)
@@ -141,5 +142,5 @@ class LightningAttention(Part):
         normed = ops.scratch("lin_normed", (T, VD), ops.act_dtype)
         with ops.section("lin_norm"):
             ops.group_rmsnorm(o, self.norm_w, self.eps, 1, normed, gate=gate, gate_kind="sigmoid_after")
-        with ops.section("wo"):
+        with ops.section("lin_wo"):
             ops.gemm(normed, self.w_o, x, accumulate=True, defer=True)

@@ -149,7 +149,8 @@ def test_state_space_recurrence_in_portions(ops32, H, G, N, P):
         ops32.linear_scan(cat(C, G * N), cat(B, G * N), cat(x, H * P), G, N, H, P, state, step, y, step_size=step_size,
                           step_bias=dev(dt_bias), a_log=dev(A_log), skip=dev(D))
         return y.cpu().numpy()
-    got = scan_in_portions(ops32, x, B, C, cuts, slots, H * N * P + 3, call)
+    assert ops32.scan_state_floats(H, N, P) == ops32.lib.hfa_linear_scan_state_floats(H, N, P) >= H * N * P
+    got = scan_in_portions(ops32, x, B, C, cuts, slots, ops32.scan_state_floats(H, N, P) + 3, call)
     for s in range(3):
         scale = np.max(np.abs(want[s]))
         assert np.max(np.abs(got[s] - want[s])) <= 2e-5 * scale, f"request {s}"
@@ -181,7 +182,8 @@ def test_linear_attention_recurrence_in_portions(ops32, dtype, H, D, Dv):
         y = torch.empty((step.n_tokens, H * Dv), dtype=torch.float32, device="cuda")
         ops32.linear_scan(qkv[:, :H * D], qkv[:, H * D:2 * H * D], qkv[:, 2 * H * D:], H, D, H, Dv, state, step, y, decay=dev(decay))
         return y.cpu().numpy()
-    got = scan_in_portions(ops32, q, k, v, cuts, slots, H * D * Dv, call)
+    assert ops32.scan_state_floats(H, D, Dv) == ops32.lib.hfa_linear_scan_state_floats(H, D, Dv) >= H * D * Dv
+    got = scan_in_portions(ops32, q, k, v, cuts, slots, ops32.scan_state_floats(H, D, Dv), call)
     for s in range(2):
         assert np.max(np.abs(got[s] - want[s])) <= 2e-5 * np.max(np.abs(want[s])), f"request {s}"
 

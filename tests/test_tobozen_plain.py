@@ -189,6 +189,7 @@ def test_values_are_mixed_with_the_first_mixing_layers(small):
 def test_configuration_and_plan():
     import hf_cpu_amd
     from hf_cpu_amd.config import config_from_dict
+    from hf_cpu_amd.kernels.ops import Ops
     from hf_cpu_amd.parts.base import FixedState, PagedKV
     for name, cfg in th.CONFIGS.items():
         c = config_from_dict(cfg)
@@ -203,10 +204,11 @@ def test_configuration_and_plan():
             if lc["type"] == "attention":
                 assert need == PagedKV(m["kv_heads"] * m["dim"], m["kv_heads"] * m["vdim"])
             elif lc["type"] == "lightning":
-                assert need == FixedState(m["heads"] * m["dim"] * m["vdim"])
+                assert need == FixedState(Ops.scan_state_floats(m["heads"], m["dim"], m["vdim"]))
+                assert need.n_floats >= m["heads"] * m["dim"] * m["vdim"]
             else:
                 channels = m["heads"] * m["vdim"] + 2 * m["groups"] * m["state"]
-                assert need == FixedState(m["heads"] * m["state"] * m["vdim"] + (m["conv"] - 1) * channels)
+                assert need == FixedState(Ops.scan_state_floats(m["heads"], m["state"], m["vdim"]) + (m["conv"] - 1) * channels)
         mixes = [lay.mixer.v_mix for lay in model.layers if hasattr(lay.mixer, "v_mix")]
         assert [v for v in mixes if v] == ["first"] + ["blend"] * (len([v for v in mixes if v]) - 1)
 
