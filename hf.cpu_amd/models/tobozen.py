@@ -15,8 +15,9 @@ EXPERT_ALPHA = 1.702          # an expert's gate half is g sigmoid(1.702 g)
 EXPERT_SHIFT = 1.0            # and its up half enters as u + 1
 
 
-def _norm(cfg, name):
-    return PartSpec("group_rmsnorm", dict(size=cfg.width, eps=cfg.norm_eps, groups=cfg.norm_groups, weight="", prefix=name))
+def _norm(cfg, name, optional=False):
+    return PartSpec("group_rmsnorm", dict(size=cfg.width, eps=cfg.norm_eps, groups=cfg.norm_groups, weight="", prefix=name,
+                                          optional=optional))
 
 
 def tobozen_plan(cfg):
@@ -47,7 +48,9 @@ def tobozen_plan(cfg):
                 prefix=prefix + "mix.", names=dict(q="q", k="k", v="v", g="g", norm="norm", o="o")))
         parts = dict(norm1=_norm(cfg, prefix + "norm1"), mixer=mixer)
         f = lc.mlp
-        if f is not None:
+        if f is None:
+            parts["norm2"] = _norm(cfg, prefix + "norm2", optional=True)      # never run; a file may hold its weight all the same
+        else:
             parts["norm2"] = _norm(cfg, prefix + "norm2")
             parts["feed_forward"] = PartSpec("moe", dict(
                 hidden_size=E, expert_size=f.ff, n_experts=f.experts, top=f.top, n_groups=1, keep_groups=1, scoring="sigmoid",

@@ -63,11 +63,13 @@ class LayerNorm(Part):
 class GroupRMSNorm(Part):
     """The vector is cut into ``groups`` equal consecutive runs; each is divided by ``sqrt(mean(run^2) + eps)`` of its
     own, and the whole is multiplied by the weight. Sums in fp32. ``weight`` is the suffix of the tensor's name after
-    ``prefix``. One group is the plain RMS norm (as a kernel of its own: nothing is left to the products around it)."""
+    ``prefix``. One group is the plain RMS norm (as a kernel of its own: nothing is left to the products around it).
+    ``optional``: the tensor may be absent (a norm that a layer's arrangement never runs)."""
     graph_safe = True
 
-    def __init__(self, size, eps, groups=1, weight="weight", prefix=""):
+    def __init__(self, size, eps, groups=1, weight="weight", prefix="", optional=False):
         super().__init__(prefix)
+        self.optional = bool(optional)
         if groups <= 0 or size % groups:
             fail(EINVAL, f"group_rmsnorm: {size} values do not form {groups} equal runs")
         self.size, self.eps, self.groups = size, float(eps), int(groups)
@@ -75,10 +77,10 @@ class GroupRMSNorm(Part):
         self.weight = None
 
     def param_specs(self):
-        return [ParamSpec(self.weight_name, (self.size,), "vector", ("one_plus_normal", 0.1))]
+        return [ParamSpec(self.weight_name, (self.size,), "vector", ("one_plus_normal", 0.1), optional=self.optional)]
 
     def bind(self, params, ops):
-        self.weight = params[self.weight_name]
+        self.weight = params.get(self.weight_name) if self.optional else params[self.weight_name]
 
     def forward(self, ops, x, out, rows=None):
         ops.group_rmsnorm(x, self.weight, self.eps, self.groups, out, rows)
