@@ -186,7 +186,9 @@ int hfa_softcap(float* x, int ld, int n_rows, int width, float cap, hipStream_t 
 // *n_tiles on the device). hfa_moe_gemm: for every row r of the plan, out[o(r), :] = act(a[s(r), :] . w[e(r)]^T)
 // (* pair_scale[pair] if given); w is [n_experts][N][K] (bf16, or fp32 beside activations of either type); s(r) = row_pair[r] / a_div if a_div > 0 else r; o(r) =
 // row_pair[r] if out_by_pair else r. tile_rows must be what hfa_moe_tile_rows gave for the plan.
-// hfa_moe_combine: x[t, :] += sum_k y[t * top + k, :].
+// hfa_moe_combine: x[t, :] += sum_k y[t * top + k, :]. `gated` 1 (N a multiple of 64, act 0): w's rows come in blocks of 32 gate rows
+// and 32 up rows, out has N / 2 columns, and with c = pair_scale of the row's pair (null: 1), g = min(c gate, limit), u = clamp(c up,
+// -limit, limit) (limit <= 0: unbounded): out = g sigmoid(alpha g) (u + shift), formed from the 32-bit sums in the product's last lines.
 int hfa_moe_route(const float* logits, int ld, int n_tokens, int n_experts, int top, int n_groups, int keep,
                   int scoring, int renorm, float out_scale, int* ids, float* weights, hipStream_t stream);
 int hfa_moe_plan(const int* ids, int n_pairs, int n_experts, int tile_rows, int* row_pair, int* tiles, int* n_tiles,
@@ -194,12 +196,14 @@ int hfa_moe_plan(const int* ids, int n_pairs, int n_experts, int tile_rows, int*
 int hfa_moe_tile_rows(int dtype, int w_dtype, int n_pairs, int n_experts, int N, int K);
 int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const void* w, int w_dtype, const int* row_pair, const int* tiles,
                  const int* n_tiles, int max_tiles, int tile_rows, void* out, int ldo, int out_dtype, int out_by_pair,
-                 const float* pair_scale, int act, int N, int K, int force_plain, hipStream_t stream);
+                 const float* pair_scale, int act, int N, int K, int force_plain, int gated, float gate_alpha, float gate_limit,
+                 float gate_shift, hipStream_t stream);
 int hfa_moe_combine(const float* y, float* x, int n_tokens, int top, int width, hipStream_t stream);
 // Gated experts: row r of the expert-ordered rows holds [gate: F | up: F] fp32 sums; with c = pair_scale[row_pair[r]]
 // (null: 1), g = min(c gate, limit), u = clamp(c up, -limit, limit) (limit <= 0: unbounded): out[r, f] = g sigmoid(alpha g) (u + shift).
+// `interleaved`: the row holds blocks of 32 gate sums and 32 up sums instead.
 int hfa_moe_gated_act(const float* gu, int ld, const int* row_pair, const float* pair_scale, void* out, int out_dtype, int ldo,
-                      int n_rows, int F, float alpha, float limit, float shift, hipStream_t stream);
+                      int n_rows, int F, float alpha, float limit, float shift, int interleaved, hipStream_t stream);
 
 // out[t, i] = silu(gate_up[t, i]) * gate_up[t, width + i].  (src/model.c:532-538)
 int hfa_swiglu(const void* gate_up, void* out, int dtype, int n_tokens, int width, hipStream_t stream);

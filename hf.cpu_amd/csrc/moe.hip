@@ -163,6 +163,21 @@ extern "C" int hfa_moe_plan(const int* ids, int n_pairs, int n_experts, int tile
 }
 
 // ---- the experts' products ----------------------------------------------------------------
+// Gated experts (`gated` in the kernels below): the rows of an expert's matrix come in blocks of 32 gate rows, 32 up rows,
+// and a product's last lines form, from the two 32-bit sums of a pair of such blocks, g sigmoid(alpha g) (u + shift) with
+// g = min(c gate, limit), u = clamp(c up, -limit, limit) (limit <= 0: unbounded), c the row's pair_scale (null: 1):
+// scaling the sums is scaling the expert's input. The output then has N / 2 columns.
+struct GatedAct { float alpha, limit, shift; };
+__device__ __forceinline__ float gated_apply(float g, float u, float c, const GatedAct ga) {
+    g *= c;
+    u *= c;
+    if (ga.limit > 0.f) {
+        g = fminf(g, ga.limit);
+        u = fminf(fmaxf(u, -ga.limit), ga.limit);
+    }
+    return g / (1.0f + expf(-ga.alpha * g)) * (u + ga.shift);
+}
+
 // Plain form, any dtype and shape: a tile of up to 32 rows x 64 columns a block, operands staged through LDS 32 k at a
 // time, every output summed over k in ascending order by one thread.
 #define PM 32
@@ -172,10 +187,11 @@ template <typename T, typename TW, typename TO>
 __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
     const T* __restrict__ a, int lda, int a_div, const TW* __restrict__ w, const int* __restrict__ row_pair,
     const int* __restrict__ tiles, const int* __restrict__ n_tiles, TO* __restrict__ out, int ldo, int out_by_pair,
-    const float* __restrict__ pair_scale, int act, int N, int K) {
+    const float* __restrict__ pair_scale, int act, int N, int K, int gated, GatedAct ga) {
     if ((int)blockIdx.x >= *n_tiles) return;
     __shared__ float a_s[PM][PK + 1];
     __shared__ float w_s[PN][PK + 1];
+    __shared__ float o_s[PM][PN + 1];
     __shared__ int src_s[PM], pair_s[PM];
     const int e = tiles[3 * blockIdx.x], r0 = tiles[3 * blockIdx.x + 1], nr = tiles[3 * blockIdx.x + 2];
     const int n0 = blockIdx.y * PN, tid = threadIdx.x;
@@ -208,6 +224,19 @@ __global__ __launch_bounds__(256) void moe_gemm_plain_kernel(
         }
         __syncthreads();
     }
+    if (gated) {                                            // columns c and c + 32 of the tile are gate and up of one output
+#pragma unroll
+        for (int i = 0; i < 8; i++) o_s[rg * 8 + i][col] = acc[i];
+        __syncthreads();
+        for (int i = tid; i < PM * (PN / 2); i += 256) {
+            const int r = i / (PN / 2), c = i % (PN / 2);
+            if (r >= nr || n0 + 32 + c >= N) continue;
+            const float sc = pair_scale ? pair_scale[pair_s[r]] : 1.f;
+            const size_t orow = out_by_pair ? (size_t)pair_s[r] : (size_t)(r0 + r);
+            out[orow * ldo + n0 / 2 + c] = from_f32<TO>(gated_apply(o_s[r][c], o_s[r][c + 32], sc, ga));
+        }
+        return;
+    }
     if (n0 + col >= N) return;
 #pragma unroll
     for (int i = 0; i < 8; i++) {
@@ -235,53 +264,73 @@ union MFrag {
 // work is cut small: a block owns 32 rows x 32 columns of one expert, its four waves take a quarter of K each (K a
 // multiple of 64) with the loads of four steps on their way at a time, and the four partial tiles are added in LDS in
 // wave order.
-template <typename TO>
+template <typename TO, bool GATED>
 __global__ __launch_bounds__(256) void moe_gemm_split_kernel(
     const uint16_t* __restrict__ a, int lda, int a_div, const uint16_t* __restrict__ w, const int* __restrict__ row_pair,
     const int* __restrict__ tiles, const int* __restrict__ n_tiles, TO* __restrict__ out, int ldo, int out_by_pair,
-    const float* __restrict__ pair_scale, int act, int N, int K) {
+    const float* __restrict__ pair_scale, int act, int N, int K, GatedAct ga) {
     if ((int)blockIdx.x >= *n_tiles) return;
-    __shared__ float part_s[4][32 * 33];
+    constexpr int NB = GATED ? 2 : 1;                       // gated: a block owns a block of 32 gate rows and its 32 up rows
+    __shared__ float part_s[4][NB][32 * 33];
     const int e = tiles[3 * blockIdx.x], r0 = tiles[3 * blockIdx.x + 1], nr = tiles[3 * blockIdx.x + 2];
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1), col = lane & 31, half = lane >> 5;
-    const int n0 = blockIdx.y * 32;
+    const int n0 = blockIdx.y * 32 * NB;
     const int row = r0 + (col < nr ? col : 0);
     const int src = a_div > 0 ? row_pair[row] / a_div : row;
     const int kq = K / 4, k0 = wave * kq;
     const uint16_t* ap = a + (size_t)src * lda + k0 + half * 8;
-    int n = n0 + col;
-    n = n < N ? n : N - 1;
-    const uint16_t* wp = w + ((size_t)e * N + n) * K + k0 + half * 8;
-    mfloatx16 acc;
+    const uint16_t* wp[NB];
 #pragma unroll
-    for (int r = 0; r < 16; r++) acc[r] = 0.f;
+    for (int b = 0; b < NB; b++) {
+        int n = n0 + 32 * b + col;
+        n = n < N ? n : N - 1;
+        wp[b] = w + ((size_t)e * N + n) * K + k0 + half * 8;
+    }
+    mfloatx16 acc[NB];
+#pragma unroll
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) acc[b][r] = 0.f;
     int k = 0;
     for (; k + 64 <= kq; k += 64) {
-        MFrag af[4], wf[4];
+        MFrag af[4], wf[NB][4];
 #pragma unroll
         for (int u = 0; u < 4; u++) {
-            wf[u].u = *reinterpret_cast<const uint4*>(wp + k + 16 * u);
+#pragma unroll
+            for (int b = 0; b < NB; b++) wf[b][u].u = *reinterpret_cast<const uint4*>(wp[b] + k + 16 * u);
             af[u].u = *reinterpret_cast<const uint4*>(ap + k + 16 * u);
         }
 #pragma unroll
-        for (int u = 0; u < 4; u++) acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[u].v, wf[u].v, acc, 0, 0, 0);
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int b = 0; b < NB; b++) acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[u].v, wf[b][u].v, acc[b], 0, 0, 0);
     }
     for (; k < kq; k += 16) {
         MFrag af, wf;
-        wf.u = *reinterpret_cast<const uint4*>(wp + k);
         af.u = *reinterpret_cast<const uint4*>(ap + k);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af.v, wf.v, acc, 0, 0, 0);
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            wf.u = *reinterpret_cast<const uint4*>(wp[b] + k);
+            acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af.v, wf.v, acc[b], 0, 0, 0);
+        }
     }
 #pragma unroll
-    for (int r = 0; r < 16; r++) part_s[wave][(8 * (r / 4) + 4 * half + (r % 4)) * 33 + col] = acc[r];
+    for (int b = 0; b < NB; b++)
+#pragma unroll
+        for (int r = 0; r < 16; r++) part_s[wave][b][(8 * (r / 4) + 4 * half + (r % 4)) * 33 + col] = acc[b][r];
     __syncthreads();
     for (int i = threadIdx.x; i < 32 * 32; i += 256) {
         const int r = i >> 5, c = i & 31;
-        if (r >= nr || n0 + c >= N) continue;
-        const float v = ((part_s[0][r * 33 + c] + part_s[1][r * 33 + c]) + part_s[2][r * 33 + c]) + part_s[3][r * 33 + c];
+        if (r >= nr || n0 + 32 * (NB - 1) + c >= N) continue;
+        float v[NB];
+#pragma unroll
+        for (int b = 0; b < NB; b++)
+            v[b] = ((part_s[0][b][r * 33 + c] + part_s[1][b][r * 33 + c]) + part_s[2][b][r * 33 + c]) + part_s[3][b][r * 33 + c];
         const int pair = (out_by_pair || pair_scale) ? row_pair[r0 + r] : 0;
         const size_t orow = out_by_pair ? (size_t)pair : (size_t)(r0 + r);
-        out[orow * ldo + n0 + c] = from_f32<TO>(hfa_act_apply(act, v) * (pair_scale ? pair_scale[pair] : 1.f));
+        const float sc = pair_scale ? pair_scale[pair] : 1.f;
+        if (GATED) out[orow * ldo + n0 / 2 + c] = from_f32<TO>(gated_apply(v[0], v[NB - 1], sc, ga));
+        else out[orow * ldo + n0 + c] = from_f32<TO>(hfa_act_apply(act, v[0]) * sc);
     }
 }
 
@@ -289,7 +338,7 @@ template <int RM, int CN, typename TO>
 __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
     const uint16_t* __restrict__ a, int lda, int a_div, const uint16_t* __restrict__ w, const int* __restrict__ row_pair,
     const int* __restrict__ tiles, const int* __restrict__ n_tiles, TO* __restrict__ out, int ldo, int out_by_pair,
-    const float* __restrict__ pair_scale, int act, int N, int K) {
+    const float* __restrict__ pair_scale, int act, int N, int K, int gated, GatedAct ga) {
     if ((int)blockIdx.x >= *n_tiles) return;
     const int e = tiles[3 * blockIdx.x], r0 = tiles[3 * blockIdx.x + 1], nr = tiles[3 * blockIdx.x + 2];
     const int wave = threadIdx.x / WAVE, lane = threadIdx.x & (WAVE - 1), col = lane & 31, half = lane >> 5;
@@ -339,6 +388,11 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(
             const int pair = (out_by_pair || pair_scale) ? row_pair[r0 + row] : 0;
             const float sc = pair_scale ? pair_scale[pair] : 1.f;
             const size_t orow = out_by_pair ? (size_t)pair : (size_t)(r0 + row);
+            if (gated) {                                    // (CN is 2: a wave's two blocks of 32 columns are gate and up)
+                if (n0 + 32 * (CN - 1) + col < N)
+                    out[orow * ldo + n0 / 2 + col] = from_f32<TO>(gated_apply(acc[i][0][r], acc[i][CN - 1][r], sc, ga));
+                continue;
+            }
 #pragma unroll
             for (int j = 0; j < CN; j++) {
                 const int n = n0 + 32 * j + col;
@@ -358,7 +412,7 @@ template <int BM, int BN, int BK, int WM, int WN, typename TO>
 __global__ __launch_bounds__(WM * WN * WAVE) void moe_gemm_lds_kernel(
     const uint16_t* __restrict__ a, int lda, int a_div, const uint16_t* __restrict__ w, const int* __restrict__ row_pair,
     const int* __restrict__ tiles, const int* __restrict__ n_tiles, TO* __restrict__ out, int ldo, int out_by_pair,
-    const float* __restrict__ pair_scale, int act, int N, int K, int n_col_tiles) {
+    const float* __restrict__ pair_scale, int act, int N, int K, int n_col_tiles, int gated, GatedAct ga) {
     constexpr int STRIDE = BK + 8, NT = WM * WN * WAVE, CPR = BK / 8, A_CH = BM * CPR / NT, W_CH = BN * CPR / NT;
     constexpr int TM = BM / WM, TN = BN / WN, FM = TM / 32, FN = TN / 32, STAGE = (BM + BN) * STRIDE;
     static_assert(BM * CPR % NT == 0 && BN * CPR % NT == 0 && TM % 32 == 0 && TN % 32 == 0, "tiles spread evenly");
@@ -471,6 +525,15 @@ __global__ __launch_bounds__(WM * WN * WAVE) void moe_gemm_lds_kernel(
             const int pair = pair_s[row];
             const float sc = pair_scale ? pair_scale[pair] : 1.f;
             const size_t orow = out_by_pair ? (size_t)pair : (size_t)(r0 + row);
+            if (gated) {                                    // (FN is even: blocks 2 j and 2 j + 1 of a wave's columns are gate and up)
+#pragma unroll
+                for (int j = 0; j + 1 < FN; j += 2) {
+                    const int nb = n0 + wn * TN + 32 * j;              // a multiple of 64: TN is
+                    if (nb + 32 + (lane & 31) < N)
+                        out[orow * ldo + nb / 2 + (lane & 31)] = from_f32<TO>(gated_apply(acc[i][j][r], acc[i][j + 1][r], sc, ga));
+                }
+                continue;
+            }
 #pragma unroll
             for (int j = 0; j < FN; j++) {
                 const int n = n0 + wn * TN + 32 * j + (lane & 31);
@@ -489,9 +552,11 @@ extern "C" int hfa_moe_tile_rows(int dtype, int w_dtype, int n_pairs, int n_expe
 extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const void* w, int w_dtype, const int* row_pair,
                             const int* tiles, const int* n_tiles, int max_tiles, int tile_rows, void* out, int ldo,
                             int out_dtype, int out_by_pair, const float* pair_scale, int act, int N, int K,
-                            int force_plain, hipStream_t stream) {
-    HFA_REQUIRE(a && w && row_pair && tiles && n_tiles && out && max_tiles > 0 && N > 0 && K > 0 && lda >= K && ldo >= N,
-                "moe_gemm: bad arguments");
+                            int force_plain, int gated, float gate_alpha, float gate_limit, float gate_shift, hipStream_t stream) {
+    HFA_REQUIRE(a && w && row_pair && tiles && n_tiles && out && max_tiles > 0 && N > 0 && K > 0 && lda >= K &&
+                    ldo >= (gated ? N / 2 : N), "moe_gemm: bad arguments");
+    HFA_REQUIRE(!gated || (N % 64 == 0 && act == 0), "moe_gemm: gated experts come in blocks of 32 gate rows and 32 up rows, without another activation");
+    const GatedAct ga = {gate_alpha, gate_limit, gate_shift};
     HFA_REQUIRE((dtype == HFA_F32 || dtype == HFA_BF16) && (out_dtype == HFA_F32 || out_dtype == HFA_BF16) &&
                     (w_dtype == HFA_F32 || w_dtype == HFA_BF16), "moe_gemm: unknown dtype");
     HFA_REQUIRE(act >= 0 && act <= HFA_ACT_LAST && a_div >= 0, "moe_gemm: bad activation or divisor");
@@ -515,24 +580,24 @@ extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const 
             configured = true;                                                                                            \
         }                                                                                                                 \
         kernel<<<grid, WM * WN * WAVE, SMEM, stream>>>((const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles, n_tiles,     \
-                                                       (TO*)out, ldo, out_by_pair, pair_scale, act, N, K, n_col_tiles);   \
+                                                       (TO*)out, ldo, out_by_pair, pair_scale, act, N, K, n_col_tiles, gated, ga);   \
     } while (0)
         if (tile_rows == 128) { if (out_dtype == HFA_F32) MOE_LDS(128, 128, 32, 2, 2, float); else MOE_LDS(128, 128, 32, 2, 2, bf16); }
         else { if (out_dtype == HFA_F32) MOE_LDS(64, 128, 32, 2, 2, float); else MOE_LDS(64, 128, 32, 2, 2, bf16); }
 #undef MOE_LDS
     } else if (mfma && K % 64 == 0) {
-        dim3 grid(max_tiles, (N + 31) / 32);
-        if (out_dtype == HFA_F32)
-            moe_gemm_split_kernel<float><<<grid, 256, 0, stream>>>((const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles,
-                                                                   n_tiles, (float*)out, ldo, out_by_pair, pair_scale, act, N, K);
-        else
-            moe_gemm_split_kernel<bf16><<<grid, 256, 0, stream>>>((const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles,
-                                                                  n_tiles, (bf16*)out, ldo, out_by_pair, pair_scale, act, N, K);
+        dim3 grid(max_tiles, gated ? N / 64 : (N + 31) / 32);
+#define MOE_SPLIT(TO, GATED)                                                                                              \
+    moe_gemm_split_kernel<TO, GATED><<<grid, 256, 0, stream>>>((const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles, \
+                                                               n_tiles, (TO*)out, ldo, out_by_pair, pair_scale, act, N, K, ga)
+        if (out_dtype == HFA_F32) { if (gated) MOE_SPLIT(float, true); else MOE_SPLIT(float, false); }
+        else { if (gated) MOE_SPLIT(bf16, true); else MOE_SPLIT(bf16, false); }
+#undef MOE_SPLIT
     } else if (mfma) {
-        const int cn = N % 256 == 0 && N >= 512 ? 2 : 1;
+        const int cn = gated || (N % 256 == 0 && N >= 512) ? 2 : 1;
         dim3 grid(max_tiles, (N + 128 * cn - 1) / (128 * cn));
 #define MOE_ARGS (const uint16_t*)a, lda, a_div, (const uint16_t*)w, row_pair, tiles, n_tiles
-#define MOE_TAIL ldo, out_by_pair, pair_scale, act, N, K
+#define MOE_TAIL ldo, out_by_pair, pair_scale, act, N, K, gated, ga
 #define MOE_GO(RM, CN)                                                                                                  \
     do {                                                                                                                \
         if (out_dtype == HFA_F32) moe_gemm_mfma_kernel<RM, CN, float><<<grid, 256, 0, stream>>>(MOE_ARGS, (float*)out, MOE_TAIL); \
@@ -547,7 +612,7 @@ extern "C" int hfa_moe_gemm(const void* a, int lda, int dtype, int a_div, const 
         dim3 grid(max_tiles, (N + PN - 1) / PN);
 #define MOE_PLAIN(TA, TW, TO)                                                                                          \
     moe_gemm_plain_kernel<TA, TW, TO><<<grid, 256, 0, stream>>>((const TA*)a, lda, a_div, (const TW*)w, row_pair, tiles, n_tiles, \
-                                                                  (TO*)out, ldo, out_by_pair, pair_scale, act, N, K)
+                                                                  (TO*)out, ldo, out_by_pair, pair_scale, act, N, K, gated, ga)
         if (dtype == HFA_F32 && w_dtype == HFA_F32 && out_dtype == HFA_F32) MOE_PLAIN(float, float, float);
         else if (dtype == HFA_BF16 && w_dtype == HFA_BF16 && out_dtype == HFA_F32) MOE_PLAIN(bf16, bf16, float);
         else if (dtype == HFA_BF16 && w_dtype == HFA_BF16 && out_dtype == HFA_BF16) MOE_PLAIN(bf16, bf16, bf16);
@@ -600,15 +665,17 @@ extern "C" int hfa_moe_combine(const float* y, float* x, int n_tokens, int top, 
 // ---- gated experts ------------------------------------------------------------------------
 // Row r of the expert-ordered rows holds [gate: F | up: F] fp32 sums of one (token, choice) pair. With c = pair_scale of
 // the row's pair (null: 1), g = min(c gate, limit), u = clamp(c up, -limit, limit) (limit <= 0: no bounds):
-// mid[r, f] = g sigmoid(alpha g) (u + shift). Scaling the sums is scaling the expert's input.
+// mid[r, f] = g sigmoid(alpha g) (u + shift). Scaling the sums is scaling the expert's input. `interleaved`: the row holds
+// blocks of 32 gate sums and 32 up sums instead (F a multiple of 32).
 template <typename TO>
 __global__ void moe_gated_act_kernel(const float* __restrict__ gu, int ld, const int* __restrict__ row_pair,
                                      const float* __restrict__ pair_scale, TO* __restrict__ out, int ldo, int F, float alpha,
-                                     float limit, float shift, size_t total) {
+                                     float limit, float shift, int interleaved, size_t total) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (size_t)gridDim.x * blockDim.x) {
         const size_t r = i / F, f = i % F;
         const float c = pair_scale ? pair_scale[row_pair[r]] : 1.f;
-        float g = c * gu[r * ld + f], u = c * gu[r * ld + F + f];
+        const size_t gi = interleaved ? (f / 32) * 64 + f % 32 : f, ui = interleaved ? gi + 32 : F + f;
+        float g = c * gu[r * ld + gi], u = c * gu[r * ld + ui];
         if (limit > 0.f) {
             g = fminf(g, limit);
             u = fminf(fmaxf(u, -limit), limit);
@@ -619,15 +686,16 @@ __global__ void moe_gated_act_kernel(const float* __restrict__ gu, int ld, const
 
 extern "C" int hfa_moe_gated_act(const float* gu, int ld, const int* row_pair, const float* pair_scale, void* out,
                                  int out_dtype, int ldo, int n_rows, int F, float alpha, float limit, float shift,
-                                 hipStream_t stream) {
-    HFA_REQUIRE(gu && out && n_rows > 0 && F > 0 && ld >= 2 * F && ldo >= F && (!pair_scale || row_pair), "moe_gated_act: bad arguments");
+                                 int interleaved, hipStream_t stream) {
+    HFA_REQUIRE(gu && out && n_rows > 0 && F > 0 && ld >= 2 * F && ldo >= F && (!pair_scale || row_pair) && (!interleaved || F % 32 == 0),
+                "moe_gated_act: bad arguments");
     HFA_REQUIRE(out_dtype == HFA_F32 || out_dtype == HFA_BF16, "moe_gated_act: unknown dtype %d", out_dtype);
     const size_t total = (size_t)n_rows * F;
     const int blocks = (int)((total + 255) / 256 < 65535 ? (total + 255) / 256 : 65535);
     if (out_dtype == HFA_F32)
-        moe_gated_act_kernel<float><<<blocks, 256, 0, stream>>>(gu, ld, row_pair, pair_scale, (float*)out, ldo, F, alpha, limit, shift, total);
+        moe_gated_act_kernel<float><<<blocks, 256, 0, stream>>>(gu, ld, row_pair, pair_scale, (float*)out, ldo, F, alpha, limit, shift, interleaved, total);
     else
-        moe_gated_act_kernel<bf16><<<blocks, 256, 0, stream>>>(gu, ld, row_pair, pair_scale, (bf16*)out, ldo, F, alpha, limit, shift, total);
+        moe_gated_act_kernel<bf16><<<blocks, 256, 0, stream>>>(gu, ld, row_pair, pair_scale, (bf16*)out, ldo, F, alpha, limit, shift, interleaved, total);
     HFA_LAUNCH_CHECK("moe_gated_act");
     return 0;
 }

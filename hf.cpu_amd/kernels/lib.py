@@ -26,7 +26,7 @@ _SIGNATURES = {
     "hfa_qkv_prepare": [P, I, I, P, P, I, I, I, I, I, I, P, P, F, P, P, P, P, P, P, I, I, P],
     "hfa_causal_conv": [P, I, I, P, P, I, I, P, c_size_t, P, P, I, I, P, I, I, P],
     "hfa_linear_scan": [P, I, P, I, I, I, P, I, I, I, I, I, P, P, I, I, P, P, P, P, c_size_t, P, P, I, P, I, P],
-    "hfa_moe_gated_act": [P, I, P, P, P, I, I, I, I, F, F, F, P],
+    "hfa_moe_gated_act": [P, I, P, P, P, I, I, I, I, F, F, F, I, P],
     "hfa_rope_table": [P, P, I, P, I, P],
     "hfa_decode_attention_supports": [I, I, I, I, I, I, I, I],
     "hfa_decode_attention": [P, I, P, P, P, I, P, P, I, P, P, P, I, I, P, I, I, I, I, I, I, I, F, P, c_size_t, P],
@@ -35,7 +35,7 @@ _SIGNATURES = {
     "hfa_softcap": [P, I, I, I, F, P],
     "hfa_moe_route": [P, I, I, I, I, I, I, I, I, F, P, P, P],
     "hfa_moe_plan": [P, I, I, I, P, P, P, P],
-    "hfa_moe_gemm": [P, I, I, I, P, I, P, P, P, I, I, P, I, I, I, P, I, I, I, I, P],
+    "hfa_moe_gemm": [P, I, I, I, P, I, P, P, P, I, I, P, I, I, I, P, I, I, I, I, I, F, F, F, P],
     "hfa_moe_combine": [P, P, I, I, I, P],
     "hfa_swiglu": [P, P, I, I, I, P],
     "hfa_scatter_i32": [P, P, P, I, P],

@@ -818,10 +818,12 @@ class Ops:
         ``w_down`` [E, width, F]. The pairs are put in expert order on the device, each expert's rows go through the
         two products in tiles, and the weighted results are added to ``x`` (fp32) choice by choice.
 
-        ``gated`` = (alpha, limit, shift): the experts are gated units whose weight scales their input. ``w_up`` then is
-        [E, 2F, width], an expert's gate rows before its up rows, and with ``c = weights[t, k]``, ``g = min(c Wgate h,
-        limit)``, ``u = clamp(c Wup h, -limit, limit)`` (``limit`` <= 0: unbounded) the expert gives ``Wdown (g
-        sigmoid(alpha g) (u + shift))``, unweighted; ``act`` is ignored."""
+        ``gated`` = (alpha, limit, shift, interleaved): the experts are gated units whose weight scales their input. ``w_up``
+        then is [E, 2F, width], an expert's gate rows before its up rows, or, ``interleaved`` (F a multiple of 32), in blocks of
+        32 gate rows and 32 up rows (``interleave_experts``); with ``c = weights[t, k]``, ``g = min(c Wgate h, limit)``, ``u =
+        clamp(c Wup h, -limit, limit)`` (``limit`` <= 0: unbounded) the expert gives ``Wdown (g sigmoid(alpha g) (u + shift))``,
+        unweighted; ``act`` is ignored. Interleaved, the up product's last lines form the activation from its 32-bit sums;
+        otherwise the sums pass through memory and a kernel of its own forms it."""
         self.settle()
         self._whole(h)
         self._source_changes(x)
@@ -854,25 +856,55 @@ class Ops:
         mid = self.scratch("moe_act", (n_pairs, F), h.dtype)
         y = self.scratch("moe_out", (n_pairs, W), torch.float32)
         if gated is not None:
-            alpha, limit, shift = gated
-            sums = self.scratch("moe_gate_up", (n_pairs, F_up), torch.float32)      # 32-bit sums: the weight scales them exactly
-            self._check(self.lib.hfa_moe_gemm(h.data_ptr(), _rows(h, "moe h"), code, top, w_up.data_ptr(), wcode, row_pair.data_ptr(),
-                                              tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, sums.data_ptr(), F_up, F32, 0,
-                                              None, 0, F_up, W, plain, self._stream()))
-            self._check(self.lib.hfa_moe_gated_act(sums.data_ptr(), F_up, row_pair.data_ptr(), weights.data_ptr(), mid.data_ptr(), code, F,
-                                                   n_pairs, F, float(alpha), float(limit), float(shift), self._stream()))
+            alpha, limit, shift, interleaved = gated
+            # A row or two an expert (a few decoded tokens): the experts' matrices are streamed once, by blocks that own 32 of
+            # their rows each; blocks that own a gate block and its up block are half as many and stream slower (835 against
+            # 900 us for the experts of a step of 8 tokens, 64 experts of 1,024 x 4,096; at 64 tokens 1,440 against 1,395),
+            # so there the activation stays a kernel of its own.
+            streamed = not plain and tile_rows == 32 and code == BF16 and wcode == BF16 and W % 64 == 0 and n_pairs <= 2 * E
+            if interleaved and not streamed:
+                self._check(self.lib.hfa_moe_gemm(h.data_ptr(), _rows(h, "moe h"), code, top, w_up.data_ptr(), wcode, row_pair.data_ptr(),
+                                                  tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, mid.data_ptr(), F, code, 0,
+                                                  weights.data_ptr(), 0, F_up, W, plain, 1, float(alpha), float(limit), float(shift),
+                                                  self._stream()))
+            else:
+                self._gated_in_two(h, code, top, w_up, wcode, row_pair, tiles, n_tiles, max_tiles, tile_rows, mid, weights, n_pairs,
+                                   F, F_up, W, plain, alpha, limit, shift, interleaved)
             self._check(self.lib.hfa_moe_gemm(mid.data_ptr(), F, code, 0, w_down.data_ptr(), wcode, row_pair.data_ptr(), tiles.data_ptr(),
                                               n_tiles.data_ptr(), max_tiles, tile_rows, y.data_ptr(), W, F32, 1, None, 0, W, F,
-                                              plain, self._stream()))
+                                              plain, 0, 0.0, 0.0, 0.0, self._stream()))
             self._check(self.lib.hfa_moe_combine(y.data_ptr(), x.data_ptr(), T, top, W, self._stream()))
             return
+        self._plain_experts(h, code, top, w_up, w_down, wcode, row_pair, tiles, n_tiles, max_tiles, tile_rows, mid, y, weights, act, F, W,
+                            plain, x, T)
+
+    def _gated_in_two(self, h, code, top, w_up, wcode, row_pair, tiles, n_tiles, max_tiles, tile_rows, mid, weights, n_pairs, F, F_up, W,
+                      plain, alpha, limit, shift, interleaved):
+        """The up product of gated experts as 32-bit sums, then the activation as a kernel of its own."""
+        sums = self.scratch("moe_gate_up", (n_pairs, F_up), torch.float32)      # 32-bit sums: the weight scales them exactly
+        self._check(self.lib.hfa_moe_gemm(h.data_ptr(), _rows(h, "moe h"), code, top, w_up.data_ptr(), wcode, row_pair.data_ptr(),
+                                          tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, sums.data_ptr(), F_up, F32, 0,
+                                          None, 0, F_up, W, plain, 0, 0.0, 0.0, 0.0, self._stream()))
+        self._check(self.lib.hfa_moe_gated_act(sums.data_ptr(), F_up, row_pair.data_ptr(), weights.data_ptr(), mid.data_ptr(), code, F,
+                                               n_pairs, F, float(alpha), float(limit), float(shift), 1 if interleaved else 0,
+                                               self._stream()))
+
+    def _plain_experts(self, h, code, top, w_up, w_down, wcode, row_pair, tiles, n_tiles, max_tiles, tile_rows, mid, y, weights, act, F, W,
+                       plain, x, T):
+        """Experts without a gate: the activation in the up product's last lines, the weights in the down product's."""
         self._check(self.lib.hfa_moe_gemm(h.data_ptr(), _rows(h, "moe h"), code, top, w_up.data_ptr(), wcode, row_pair.data_ptr(),
                                           tiles.data_ptr(), n_tiles.data_ptr(), max_tiles, tile_rows, mid.data_ptr(), F, code, 0, None,
-                                          self.ACTIVATIONS[act], F, W, plain, self._stream()))
+                                          self.ACTIVATIONS[act], F, W, plain, 0, 0.0, 0.0, 0.0, self._stream()))
         self._check(self.lib.hfa_moe_gemm(mid.data_ptr(), F, code, 0, w_down.data_ptr(), wcode, row_pair.data_ptr(), tiles.data_ptr(),
                                           n_tiles.data_ptr(), max_tiles, tile_rows, y.data_ptr(), W, F32, 1, weights.data_ptr(), 0, W, F,
-                                          plain, self._stream()))
+                                          plain, 0, 0.0, 0.0, 0.0, self._stream()))
         self._check(self.lib.hfa_moe_combine(y.data_ptr(), x.data_ptr(), T, top, W, self._stream()))
+
+    @staticmethod
+    def interleave_experts(w_gate, w_up):
+        """[E, 2F, width] from [E, F, width] twice: of every expert rows 0..31 of gate, rows 0..31 of up, rows 32..63 of gate, ..."""
+        E, F, W = w_gate.shape
+        return torch.stack([w_gate.view(E, F // 32, 32, W), w_up.view(E, F // 32, 32, W)], dim=2).reshape(E, 2 * F, W).contiguous()
 
     def scatter_i32(self, dst, idx, val):
         n = idx.numel()

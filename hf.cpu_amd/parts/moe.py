@@ -24,7 +24,8 @@ class MixtureOfExperts(Part):
     ``gated`` = dict(alpha, limit, shift): the experts are gated units, ``Wdown (g sigmoid(alpha g) (u + shift))`` with
     ``g = min(Wgate h', limit)``, ``u = clamp(Wup h', -limit, limit)`` (``limit`` <= 0: unbounded), and ``h' = weight_e h``:
     the weight scales the expert's input, not its output (``weight_on="input"``). The gate matrices are named by
-    ``names["gate"]``; gate and up of an expert are held as one matrix, gate rows first."""
+    ``names["gate"]``; gate and up of an expert are held as one matrix: in blocks of 32 gate rows and 32 up rows where the
+    expert's size is a multiple of 32 (the up product then forms the activation in its last lines), else gate rows first."""
     graph_safe = True
 
     def __init__(self, hidden_size, expert_size, n_experts, top, n_groups=1, keep_groups=1, activation="relu2",
@@ -33,7 +34,8 @@ class MixtureOfExperts(Part):
         super().__init__(prefix)
         if weight_on not in ("output", "input") or (weight_on == "input") != (gated is not None):
             fail(ENOTSUP, "moe: gated experts weigh their input, experts without a gate their output; other pairings are not implemented")
-        self.gated = None if gated is None else (float(gated["alpha"]), float(gated.get("limit", 0.0)), float(gated.get("shift", 0.0)))
+        self.gated = None if gated is None else (float(gated["alpha"]), float(gated.get("limit", 0.0)), float(gated.get("shift", 0.0)),
+                                                 expert_size % 32 == 0)
         self.weight_on = weight_on
         if activation not in ("gelu_erf", "gelu_tanh", "relu2"):
             fail(ENOTSUP, f"moe: activation '{activation}' is not implemented")
@@ -66,8 +68,13 @@ class MixtureOfExperts(Part):
     def bind(self, params, ops):
         self.w_router = params[self._name("router")]
         ups = [params.pop(self._name("up", e)) for e in range(self.n_experts)]
-        if self.gated is not None:                  # an expert's gate rows, then its up rows: one product gives both
-            ups = [torch.cat([params.pop(self._name("gate", e)), u], 0) for e, u in enumerate(ups)]
+        if self.gated is not None:                  # gate and up of an expert in one matrix: one product gives both
+            gates = [params.pop(self._name("gate", e)) for e in range(self.n_experts)]
+            if self.gated[3]:
+                ups = [ops.interleave_experts(g.unsqueeze(0), u.unsqueeze(0))[0] for g, u in zip(gates, ups)]
+            else:
+                ups = [torch.cat([g, u], 0) for g, u in zip(gates, ups)]
+            del gates
         downs = [params.pop(self._name("down", e)) for e in range(self.n_experts)]
         dt = torch.float32 if any(m.dtype == torch.float32 for m in ups + downs) else ups[0].dtype
         self.w_up = memory.cat([m.to(dt).unsqueeze(0) for m in ups], 0, f"{self.prefix}up matrices of all experts")

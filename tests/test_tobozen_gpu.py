@@ -311,7 +311,8 @@ def test_a_key_far_away_among_hundreds_and_scores_far_below_zero(ops32, ops16, d
 
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("T,W,F,E,top,limit", [(1, 40, 12, 5, 2, 0.5), (7, 256, 80, 10, 1, 1.25), (300, 256, 64, 4, 4, 2.0), (33, 128, 32, 16, 3, 7.0),
-                                               (2100, 256, 32, 8, 2, 1.0), (64, 64, 16, 1, 1, 0.25)])
+                                               (2100, 256, 32, 8, 2, 1.0), (64, 64, 16, 1, 1, 0.25), (5, 256, 96, 6, 2, 1.0),
+                                               (9, 72, 64, 3, 1, 0.5), (1200, 512, 192, 4, 2, 1.5), (40, 80, 64, 4, 2, 1.0), (700, 144, 96, 3, 1, 2.0)])
 def test_router_and_gated_experts_weighted_on_their_input(ops32, ops16, dtype, T, W, F, E, top, limit):
     """Sigmoid scores, the best experts, the scores themselves as weights, and the weight inside the expert: the
     bounds at ``limit`` cut differently for ``expert(w h)`` than for ``w expert(h)``."""
@@ -334,17 +335,22 @@ def test_router_and_gated_experts_weighted_on_their_input(ops32, ops16, dtype, T
     f = dict(expert=dict(ff=F, limit=limit), router=dict(experts=E, top=top))
     want, _ = pt.moe_ff(h, w, "", f, choices=ids_h)
     x = torch.zeros((T, W), dtype=torch.float32, device="cuda")
-    w_up = dev(np.stack([np.concatenate([w[f"e{e}.gate"], w[f"e{e}.up"]]) for e in range(E)]), dtype)
+    gates = dev(np.stack([w[f"e{e}.gate"] for e in range(E)]), dtype)
+    ups = dev(np.stack([w[f"e{e}.up"] for e in range(E)]), dtype)
     w_down = dev(np.stack([w[f"e{e}.down"] for e in range(E)]), dtype)
-    for plain_kernels in (False, True):
-        x.zero_()
-        ops.force_plain_gemm = plain_kernels
-        try:
-            ops.moe_experts(dev(h, dtype), ids, wts, w_up, w_down, None, x, gated=(1.702, limit, 1.0))
-        finally:
-            ops.force_plain_gemm = False
-        err = np.max(np.abs(x.cpu().numpy() - want)) / np.max(np.abs(want))
-        assert err <= (1e-5 if dtype == torch.float32 else 1e-2), f"plain={plain_kernels}: {err:.3e}"
+    # gate rows before up rows (the activation is a kernel of its own), and, where the size allows, in blocks of 32 and 32
+    # (the activation in the up product's last lines); the matrix-core kernels and the plain one
+    layouts = [(torch.cat([gates, ups], 1), False)] + ([(ops.interleave_experts(gates, ups), True)] if F % 32 == 0 else [])
+    for w_up, interleaved in layouts:
+        for plain_kernels in (False, True):
+            x.zero_()
+            ops.force_plain_gemm = plain_kernels
+            try:
+                ops.moe_experts(dev(h, dtype), ids, wts, w_up, w_down, None, x, gated=(1.702, limit, 1.0, interleaved))
+            finally:
+                ops.force_plain_gemm = False
+            err = np.max(np.abs(x.cpu().numpy() - want)) / np.max(np.abs(want))
+            assert err <= (1e-5 if dtype == torch.float32 else 1e-2), f"interleaved={interleaved} plain={plain_kernels}: {err:.3e}"
 
 
 # ---- whole models ---------------------------------------------------------------------------------------------------
