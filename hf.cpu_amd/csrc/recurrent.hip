@@ -192,18 +192,29 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(
         stash(g_);
         __syncthreads();
         fetch(g_, c0 + 2 * TOK);
-        auto token = [&](int t) {
-            const float a = a_s[t], bv = b_s[t] * v_s[t * PT + pl];
+        // A token's operands leave LDS two tokens before (three gained nothing) its multiply-adds: the only chain from token to token is the
+        // state's own, and a wave that has a SIMD to itself would otherwise wait for every read.
+        struct Operands { float4 k[NPT / 4], q[NPT / 4]; float a, bv; };
+        auto read = [&](int t, Operands& o) {
             const float4* kt = reinterpret_cast<const float4*>(k_s + t * NPAD + ns * NPT);
             const float4* qt = reinterpret_cast<const float4*>(q_s + t * NPAD + ns * NPT);
+#pragma unroll
+            for (int i = 0; i < NPT / 4; i++) {
+                o.k[i] = kt[i];
+                o.q[i] = qt[i];
+            }
+            o.a = a_s[t];
+            o.bv = b_s[t] * v_s[t * PT + pl];
+        };
+        auto token = [&](int t, const Operands& o) {
             float acc0 = 0.f, acc1 = 0.f;
 #pragma unroll
             for (int i = 0; i < NPT / 4; i++) {
-                const float4 kk = kt[i], qq = qt[i];
-                st[4 * i] = fmaf(a, st[4 * i], kk.x * bv);
-                st[4 * i + 1] = fmaf(a, st[4 * i + 1], kk.y * bv);
-                st[4 * i + 2] = fmaf(a, st[4 * i + 2], kk.z * bv);
-                st[4 * i + 3] = fmaf(a, st[4 * i + 3], kk.w * bv);
+                const float4 kk = o.k[i], qq = o.q[i];
+                st[4 * i] = fmaf(o.a, st[4 * i], kk.x * o.bv);
+                st[4 * i + 1] = fmaf(o.a, st[4 * i + 1], kk.y * o.bv);
+                st[4 * i + 2] = fmaf(o.a, st[4 * i + 2], kk.z * o.bv);
+                st[4 * i + 3] = fmaf(o.a, st[4 * i + 3], kk.w * o.bv);
                 acc0 = fmaf(st[4 * i], qq.x, acc0);
                 acc1 = fmaf(st[4 * i + 1], qq.y, acc1);
                 acc0 = fmaf(st[4 * i + 2], qq.z, acc0);
@@ -212,10 +223,20 @@ __global__ __launch_bounds__(SCAN_THREADS) void linear_scan_kernel(
             part_s[t * SCAN_THREADS + tid] = acc0 + acc1;
         };
         if (nt == TOK) {
-#pragma unroll 4
-            for (int t = 0; t < TOK; t++) token(t);
+            Operands ring[3];
+            read(0, ring[0]);
+            read(1, ring[1]);
+#pragma unroll
+            for (int t = 0; t < TOK; t++) {
+                if (t + 2 < TOK) read(t + 2, ring[(t + 2) % 3]);
+                token(t, ring[t % 3]);
+            }
         } else {
-            for (int t = 0; t < nt; t++) token(t);
+            for (int t = 0; t < nt; t++) {
+                Operands o;
+                read(t, o);
+                token(t, o);
+            }
         }
         __syncthreads();
         // the outputs of the tokens just walked: thread -> (token, column), the lanes' shares added in lane order
