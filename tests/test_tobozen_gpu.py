@@ -597,3 +597,26 @@ def test_a_file_may_hold_the_weights_that_are_never_read(gpu, tmp_path):
         engine = hf_cpu_amd.load_engine(d, dtype="float32", page_tokens=8, max_tokens=64, max_seqs=1)
         outs.append(engine.step([("a", toks, list(range(len(toks))))]).cpu().numpy())
     assert np.array_equal(outs[0], outs[1])
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_configurations_drawn_at_random(gpu, tmp_path, seed):
+    """Layers of any kind in any order with sizes drawn at random (even seeds: sizes for the matrix cores): a prompt, a portion
+    that starts in the middle of a page, then single tokens, in fp32 and in bf16 (with the engine's choice of experts)."""
+    import hf_cpu_amd
+    rng = np.random.default_rng(100 + seed)
+    cfg = th.random_config(rng, big=seed % 2 == 0)
+    d = th.make_model_dir(str(tmp_path / "m"), cfg, seed=seed, stored="BF16" if seed % 2 == 0 else "F32")
+    toks = [int(t) for t in rng.integers(0, cfg["vocab"], 110)]
+    pcfg, w = pt.read_model(d)
+    steps = [helpers._step(0, [("a", toks[:55], range(55))]), helpers._step(1, [("a", toks[55:88], range(33))])]
+    steps += [helpers._step(2 + i, [("a", toks[88 + i:89 + i], [0])], ["a"] if i == 21 else []) for i in range(22)]
+    for dtype in ("float32", "bfloat16"):
+        engine = hf_cpu_amd.load_engine(d, dtype=dtype, page_tokens=16, max_tokens=128, max_seqs=2, graphs=dtype == "float32")
+        if dtype == "float32":
+            got, want = helpers.run_trace_in_engine(engine, steps), pt.forward(pcfg, w, toks)
+        else:
+            with th.record_choices(engine) as rec:
+                got = helpers.run_trace_in_engine(engine, steps)
+            want = th.forward_with_choices(pcfg, w, toks, rec.chosen.get("a", {}))
+        helpers.compare(got, {"a": want}, TOL[dtype] if dtype == "float32" else 6e-2, f"random configuration {seed} {dtype}: {cfg}")

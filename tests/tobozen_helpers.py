@@ -162,3 +162,46 @@ def forward_with_choices(cfg, w, tokens, chosen, margins=None):
                 margins[(l, t)] = (float(gap), set(int(e) for e in ids[t]) == set(int(e) for e in own[t]))
         choices[l] = ids
     return pt.forward(cfg, w, tokens, choices=choices)
+
+
+def random_config(rng, big):
+    """A configuration drawn at random: two to six layers of any kind in any order, with sizes that the matrix-core kernels
+    take (``big``) or that none of them takes; layers that mix values agree on the values' width, as the design demands."""
+    def pick(*xs):
+        return xs[int(rng.integers(0, len(xs)))]
+    width = pick(128, 256, 384) if big else pick(24, 40, 56, 72, 100)
+    groups = pick(1, 2, 4)
+    layers, mixed = [], None
+    for _ in range(int(rng.integers(2, 7))):
+        kind = pick("mamba2", "attention", "lightning")
+        if kind == "mamba2":
+            H = pick(2, 4, 6, 8)
+            G = pick(*[g for g in (1, 2, 3, 4, 6, 8) if H % g == 0])
+            P = pick(16, 32, 64, 40) if big else pick(4, 5, 12, 20)
+            N = pick(16, 32, 48, 64, 128) if big else pick(3, 8, 17, 24)
+            mix = mamba2(H, P, N, G, pick(1, 2, 3, 4), pick(*[g for g in (1, 2, 4, H) if (H * P) % g == 0]))
+        elif kind == "attention":
+            G = pick(1, 2, 4)
+            H = G * pick(1, 2, 4, 7)
+            D = pick(32, 64, 128) if big else pick(6, 10, 16, 24)
+            v_mix = bool(rng.integers(0, 2))
+            if v_mix and mixed is not None and mixed % G == 0:
+                Dv = mixed // G
+            elif v_mix and mixed is not None:
+                v_mix, Dv = False, D
+            else:
+                Dv = pick(D, D // 2, 32 if big else 8)
+            if v_mix and mixed is None:
+                mixed = G * Dv
+            rot = max(2, pick(D, D // 2, 2) // 2 * 2)
+            mix = attention(H, G, D, Dv, rot, pick(100.0, 10000.0, 1e6), scale=pick(None, 0.2, 0.05), v_mix=v_mix)
+        else:
+            H = pick(1, 2, 3, 8)
+            mix = lightning(H, pick(32, 64, 128) if big else pick(5, 8, 20), pick(32, 64, 96) if big else pick(4, 12, 30),
+                            [pick(0.5, 0.75, 0.9375, 0.984375, 1.0) for _ in range(H)])
+        E = pick(1, 2, 5, 8, 16)
+        mlp = None if rng.random() < 0.25 else moe(E, int(rng.integers(1, min(E, 4) + 1)), pick(32, 64, 96, 48) if big else pick(4, 10, 24),
+                                                   pick(0.5, 1.0, 3.0, 7.0))
+        layers.append(layer(mix, mlp))
+    return dict(architecture="Tobozen", vocab=int(rng.integers(50, 400)), width=width,
+                norm=dict(eps=pick(1e-5, 1e-6), groups=groups if width % groups == 0 else 1), layers=layers)
